@@ -1,0 +1,142 @@
+"""The step function: run the tokens a step brings, from the cache, as one batch.
+
+``ModelRunner.step(entries)`` takes, for each request in the step, its next
+tokens and the places whose logits are wanted; it reserves pages, packs the
+batch, runs the model once over all tokens of all entries, records the new
+lengths and returns float32 logits ``[wanted, vocab]`` in the order of the
+entries and of their ``want`` lists. Portions of prompts and single decoded
+tokens go through the same pass (the reference's runner may split them into
+two forwards: qwen3_runtime/engine/model_runner.py:118-127; its contract is
+qwen3_runtime/engine/runner.py:27-41).
+
+Steps that are pure decoding (one token per entry) are replayed from a HIP
+graph captured per batch size, with the step's arrays copied into static
+buffers first (reference: qwen3_runtime/engine/cuda_graph.py:152-188).
+"""
+
+from __future__ import annotations
+
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from ..parts.base import GroupView, StepContext
+from .batch import PackedStep, StepEntry, pack_step
+
+
+class ModelRunner:
+    def __init__(self, model, cache, ops, *, dtype: torch.dtype, device, max_model_len: int | None = None,
+                 hip_graph: bool = False):
+        self.model = model
+        self.cache = cache
+        self.ops = ops
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.max_model_len = int(max_model_len or model.plan.max_positions)
+        self.vocab_size = model.plan.vocab_size
+        self.hip_graph = bool(hip_graph) and self.device.type == "cuda"
+        self._graphs: dict[tuple, "_DecodeGraph"] = {}
+        self._pinned: torch.Tensor | None = None
+        self.graph_max_batch = 256
+
+    # ---- public ------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
+        for e in entries:
+            end = self.cache.length(e.request_id) + len(e.tokens)
+            if end > self.max_model_len:
+                raise ValueError(
+                    f"request {e.request_id!r} would reach {end} tokens; the limit is {self.max_model_len}"
+                )
+        for e in entries:
+            self.cache.reserve(e.request_id, len(e.tokens))
+        pure_decode = all(len(e.tokens) == 1 for e in entries)
+        if self.hip_graph and pure_decode and len(entries) <= self.graph_max_batch:
+            logits = self._step_graph(entries)
+        else:
+            packed = pack_step(entries, self.cache, self.vocab_size)
+            dev = self._upload(packed)
+            logits = self._forward(packed, dev)
+        for e in entries:
+            self.cache.commit(e.request_id, len(e.tokens))
+        return logits
+
+    # ---- eager path ----------------------------------------------------------
+    def _upload(self, packed: PackedStep) -> dict[str, torch.Tensor]:
+        """All arrays of a step in one host buffer, one copy to the device."""
+        sizes = [(name, a.size) for name, a in packed.arrays.items()]
+        # keep every array 16-byte aligned on the device
+        offsets, total = [], 0
+        for _, n in sizes:
+            offsets.append(total)
+            total += (n + 3) // 4 * 4
+        total = max(total, 4)
+        if self.device.type == "cuda":
+            if self._pinned is None or self._pinned.numel() < total:
+                self._pinned = torch.empty(max(total, 1 << 16), dtype=torch.int32, pin_memory=True)
+            host = self._pinned[:total]
+        else:
+            host = torch.empty(total, dtype=torch.int32)
+        host_np = host.numpy()
+        for (name, n), off in zip(sizes, offsets):
+            host_np[off: off + n] = packed.arrays[name].reshape(-1)
+        if self.device.type == "cuda":
+            dev = torch.empty(total, dtype=torch.int32, device=self.device)
+            dev.copy_(host, non_blocking=True)
+            # the pinned buffer is rewritten by the next step: wait for the copy
+            torch.cuda.current_stream(self.device).synchronize()
+        else:
+            dev = host.clone()
+        out = {}
+        for (name, n), off in zip(sizes, offsets):
+            out[name] = dev[off: off + n].view(packed.arrays[name].shape)
+        return out
+
+    def _context(self, packed: PackedStep, dev: dict[str, torch.Tensor]) -> StepContext:
+        groups = [
+            GroupView(g.page_size, g.window, dev[f"table{gi}"], dev[f"slots{gi}"])
+            for gi, g in enumerate(self.cache.groups)
+        ]
+        return StepContext(
+            ops=self.ops,
+            dtype=self.dtype,
+            device=self.device,
+            num_tokens=packed.num_tokens,
+            num_seqs=packed.num_seqs,
+            positions=dev["positions"],
+            cu_q=dev["cu_q"],
+            kv_lens=dev["kv_lens"],
+            seq_of_token=dev["seq_of_token"],
+            state_slots=dev["state_slots"],
+            first_span=dev["first_span"],
+            q_lens_host=packed.q_lens,
+            kv_lens_host=packed.kv_lens,
+            max_q_len=max(packed.q_lens),
+            max_kv_len=max(packed.kv_lens),
+            groups=groups,
+        )
+
+    def _forward(self, packed: PackedStep, dev: dict[str, torch.Tensor]):
+        ctx = self._context(packed, dev)
+        views = [
+            None if st.cache is None else self.cache.view(st.cache, ctx.groups, st.writes_cache)
+            for st in self.model.plan.order
+        ]
+        rows = dev["rows"] if packed.num_rows else None
+        with torch.inference_mode():
+            return self.model.forward(ctx, dev["ids"], views, rows)
+
+    # ---- graph path ----------------------------------------------------------
+    def _step_graph(self, entries: Sequence[StepEntry]):
+        from .graph import DecodeGraph
+
+        max_kv = max(self.cache.length(e.request_id) + 1 for e in entries)
+        key = DecodeGraph.key_for(len(entries), max_kv, all(len(e.want) == 1 for e in entries))
+        if key is None:
+            packed = pack_step(entries, self.cache, self.vocab_size)
+            return self._forward(packed, self._upload(packed))
+        graph = self._graphs.get(key)
+        if graph is None:
+            graph = DecodeGraph(self, key)
+            self._graphs[key] = graph
+        return graph.run(entries)
