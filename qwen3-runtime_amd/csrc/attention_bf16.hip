@@ -1,0 +1,236 @@
+// Paged attention on MFMA for bfloat16, one head size per build (QRT_HEAD_DIM,
+// a multiple of 16). Serves prompt portions, single decoded tokens and batches
+// that mix both, with optional splitting of the keys across blocks.
+//
+// Rows. For one sequence and one key/value head the work is a matrix of
+// q_len * g rows, row = token * g + (query head within the group): all g query
+// heads that share a key head sit in the same tile, so a decoded token fills g
+// rows and a prompt portion fills tiles of 16 rows per wave. The host passes a
+// list of tiles (sequence, first row); blockIdx.x walks it.
+//
+// Products. Scores are formed transposed, S^T = K Q^T, with the 16x16x32 MFMA:
+// the A operand is 16 keys x 32 head elements read straight from the key page,
+// the B operand 32 head elements x 16 rows of Q held in registers. The 16 key
+// rows of the two MFMAs that cover a block of 32 keys are permuted (row
+// 4 quad + r of sub-block kb holds key 8 quad + 4 kb + r) so that each lane ends
+// up with the scores of 8 consecutive keys for its row: exactly the B operand
+// (P^T) of the second product O^T = V^T P^T, whose A operand is then 8
+// consecutive keys of one head element: one 16-byte read from the value page,
+// which stores values transposed ([page, head, D, offset]). No data crosses
+// lanes except the row maximum and sum.
+//
+// Softmax is online, float32, in base 2 (scores pre-multiplied by
+// scale * log2 e); probabilities are rounded to bfloat16 for the second
+// product, accumulation is float32. Key j is visible to the row at position p
+// iff j <= p and (no window or j > p - window).
+#include "common.h"
+#include <math.h>
+
+#ifndef QRT_HEAD_DIM
+#error "build with -DQRT_HEAD_DIM=<multiple of 16>"
+#endif
+#if QRT_HEAD_DIM % 16 != 0 || QRT_HEAD_DIM < 16 || QRT_HEAD_DIM > 512
+#error "QRT_HEAD_DIM must be a multiple of 16 between 16 and 512"
+#endif
+
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+struct AttnTileArgs {
+  const bf16_t* q;        // [T, nq * D]
+  bf16_t* out;            // [T, nq * D]
+  const bf16_t* k_cache;  // [pages, nkv, page_size, D]
+  const bf16_t* v_cache;  // [pages, nkv, D, page_size]
+  const int* cu_q;        // [S + 1]
+  const int* kv_lens;     // [S]
+  const int* block_table; // [S, table_width]
+  const int* tile_seq;    // [num_tiles]
+  const int* tile_row0;   // [num_tiles]
+  float* part_o;          // [T, nq, num_splits, D]   (num_splits > 1)
+  float* part_lse;        // [T, nq, num_splits]      base-2 log of the split's sum, -inf if empty
+  int table_width, num_tiles, nq, nkv, page_size, window, num_splits, waves;
+  float scale_log2;
+};
+
+constexpr int D = QRT_HEAD_DIM;
+constexpr int KFULL = D / 32;        // 32-wide steps of the first product
+constexpr bool KTAIL = (D % 32) != 0;  // one 16-wide step more
+constexpr int DB = D / 16;           // 16-wide blocks of the head dimension
+
+__global__ __launch_bounds__(256) void attention_bf16_kernel(AttnTileArgs a) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int seq = a.tile_seq[blockIdx.x];
+  const int kvh = blockIdx.y, split = blockIdx.z;
+  const int g = a.nq / a.nkv;
+  const int q_begin = a.cu_q[seq];
+  const int q_len = a.cu_q[seq + 1] - q_begin;
+  const int kv_len = a.kv_lens[seq];
+  const int n_rows = q_len * g;
+  const int row0 = a.tile_row0[blockIdx.x] + 16 * wave;
+  if (row0 >= n_rows) return;
+  const int first_pos = kv_len - q_len;
+  const int my_row = row0 + r16;
+  const bool row_valid = my_row < n_rows;
+  const int row_c = row_valid ? my_row : n_rows - 1;
+  const int tok = row_c / g, hg = row_c - tok * g;
+  const int qpos = first_pos + tok;
+  const int head = kvh * g + hg;
+  const int ps = a.page_size;
+  const int* table = a.block_table + (size_t)seq * a.table_width;
+
+  // Q as B operands, kept for the whole loop
+  const bf16_t* qp = a.q + ((size_t)(q_begin + tok) * a.nq + head) * D;
+  bf16x8_t qreg[KFULL > 0 ? KFULL : 1];
+#pragma unroll
+  for (int i = 0; i < KFULL; ++i) qreg[i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
+  s16x4_t qtail = {0, 0, 0, 0};
+  if (KTAIL) qtail = *(const s16x4_t*)(qp + 32 * KFULL + 4 * quad);
+
+  // keys this wave may need: [lo, pos_max]
+  const int row_last = min(row0 + 15, n_rows - 1);
+  const int pos_min = first_pos + row0 / g, pos_max = first_pos + row_last / g;
+  const int lo = a.window > 0 ? max(0, pos_min - a.window + 1) : 0;
+  const int blk_begin = lo >> 5, blk_end = (pos_max >> 5) + 1;
+  const int per = (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
+  const int b0 = blk_begin + split * per;
+  const int b1 = min(blk_end, b0 + per);
+
+  f32x4_t o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) o[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int b = b0; b < b1; ++b) {
+    const int base = b << 5;
+    f32x4_t s[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      int kidx = base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3);
+      kidx = min(max(kidx, lo), pos_max);  // stay inside pages this sequence holds; masked below
+      const int page = table[kidx / ps];
+      const bf16_t* kp = a.k_cache + (((size_t)page * a.nkv + kvh) * ps + (kidx % ps)) * D;
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < KFULL; ++i) {
+        const bf16x8_t kk = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk, qreg[i], acc, 0, 0, 0);
+      }
+      if (KTAIL) {
+        const s16x4_t kk = *(const s16x4_t*)(kp + 32 * KFULL + 4 * quad);
+        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kk, qtail, acc, 0, 0, 0);
+      }
+      s[kb] = acc;
+    }
+    // this lane: row r16, keys base + 8 quad + 4 kb + r
+    float p[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = base + 8 * quad + e;
+      const bool vis = row_valid && key <= qpos && (a.window == 0 || key > qpos - a.window);
+      p[e] = vis ? s[e >> 2][e & 3] * a.scale_log2 : -INFINITY;
+      mx = fmaxf(mx, p[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = exp2f(m - m_use);
+    float psum = 0.f;
+    bf16x8_t pb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pe = exp2f(p[e] - m_use);
+      psum += pe;
+      pb[e] = (bf16_t)pe;
+    }
+    l = l * corr + psum;
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < DB; ++i) o[i] *= corr;
+
+    // values: 8 consecutive keys base + 8 quad .. + 7 of head element 16 i + r16
+    const int kv0 = base + 8 * quad;
+    const bool vload = kv0 <= pos_max && kv0 + 7 >= lo;
+    const int vpage = vload ? table[kv0 / ps] : 0;
+    const bf16_t* vp = a.v_cache + (((size_t)vpage * a.nkv + kvh) * D + r16) * ps + (kv0 % ps);
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+      bf16x8_t vv;
+      if (vload) vv = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
+      else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vv[e] = (bf16_t)0.0f;
+      }
+      o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pb, o[i], 0, 0, 0);
+    }
+  }
+
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!row_valid) return;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  const size_t row_index = (size_t)(q_begin + tok) * a.nq + head;
+  if (a.num_splits == 1) {
+    bf16_t* op = a.out + row_index * D;
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+      bf16x4_t w;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) w[r] = (bf16_t)(o[i][r] * inv);
+      *(bf16x4_t*)(op + 16 * i + 4 * quad) = w;
+    }
+  } else {
+    float* op = a.part_o + (row_index * a.num_splits + split) * D;
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+      f32x4_t w = o[i] * inv;
+      *(f32x4_t*)(op + 16 * i + 4 * quad) = w;
+    }
+    if (quad == 0) a.part_lse[row_index * a.num_splits + split] = l > 0.f ? m + log2f(l) : -INFINITY;
+  }
+}
+
+// out[row] = sum_s 2^(lse_s - M) O_s / sum_s 2^(lse_s - M); empty splits weigh 0
+__global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
+                                       bf16_t* __restrict__ out, int num_splits) {
+  const size_t row = blockIdx.x;
+  const float* lse = part_lse + row * num_splits;
+  float mx = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, lse[s]);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float acc = 0.f, wsum = 0.f;
+    if (mx != -INFINITY) {
+      for (int s = 0; s < num_splits; ++s) {
+        const float w = exp2f(lse[s] - mx);
+        wsum += w;
+        acc += w * part_o[(row * num_splits + s) * D + d];
+      }
+    }
+    out[row * D + d] = (bf16_t)(wsum > 0.f ? acc / wsum : 0.f);
+  }
+}
+
+extern "C" int qrt_attention_bf16_head_dim() { return D; }
+
+extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, hipStream_t stream) {
+  AttnTileArgs a = *args;
+  QRT_CHECK(a.nq > 0 && a.nkv > 0 && a.nq % a.nkv == 0, "attention: %d query heads do not divide into %d key heads",
+            a.nq, a.nkv);
+  QRT_CHECK(a.page_size > 0 && a.page_size % 8 == 0,
+            "attention (bfloat16): page size %d must be a multiple of 8", a.page_size);
+  QRT_CHECK(a.waves == 1 || a.waves == 2 || a.waves == 4, "attention: waves per block must be 1, 2 or 4");
+  QRT_CHECK(a.num_splits >= 1 && a.num_splits <= 65535 && a.nkv <= 65535, "attention: bad split or head count");
+  QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse), "attention: split run without scratch");
+  QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
+  if (a.num_tiles == 0) return 0;
+  dim3 grid(a.num_tiles, a.nkv, a.num_splits), block(64 * a.waves);
+  attention_bf16_kernel<<<grid, block, 0, stream>>>(a);
+  QRT_LAUNCH_CHECK("attention_bf16");
+  if (a.num_splits > 1) {
+    attention_merge_kernel<<<dim3(num_rows_total), dim3(D >= 64 ? 64 : 32), 0, stream>>>(a.part_o, a.part_lse, a.out,
+                                                                                         a.num_splits);
+    QRT_LAUNCH_CHECK("attention_merge");
+  }
+  return 0;
+}

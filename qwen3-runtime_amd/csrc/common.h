@@ -1,0 +1,86 @@
+// Shared declarations of the HIP library (gfx950, wave64).
+//
+// Every entry point is extern "C", takes raw device pointers plus sizes and a
+// stream, validates what it can on the host, launches on that stream and
+// returns 0, or a negative code after recording a message that
+// qrt_last_error() returns. Nothing here allocates device memory.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+#define QRT_WAVE 64
+
+// dtype codes shared with the Python side
+#define QRT_F32 0
+#define QRT_BF16 1
+
+extern "C" const char* qrt_last_error();
+int qrt_fail(const char* fmt, ...);
+
+#define QRT_CHECK(cond, ...)                 \
+  do {                                       \
+    if (!(cond)) return qrt_fail(__VA_ARGS__); \
+  } while (0)
+
+#define QRT_LAUNCH_CHECK(name)                                                     \
+  do {                                                                             \
+    hipError_t e_ = hipGetLastError();                                             \
+    if (e_ != hipSuccess) return qrt_fail("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+  } while (0)
+
+template <typename T> __device__ __forceinline__ float to_f32(T x);
+template <> __device__ __forceinline__ float to_f32<float>(float x) { return x; }
+template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t x) { return (float)x; }
+
+template <typename T> __device__ __forceinline__ T from_f32(float x);
+template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return (bf16_t)x; }
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+  return x;
+}
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+  return x;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.
+// `red` is shared memory of at least 17 floats. Order of additions is fixed.
+__device__ __forceinline__ float block_sum(float x, float* red) {
+  x = wave_sum(x);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = x;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = 0.f;
+    for (int i = 0; i < nw; ++i) s += red[i];
+    red[16] = s;
+  }
+  __syncthreads();
+  return red[16];
+}
+__device__ __forceinline__ float block_max(float x, float* red) {
+  x = wave_max(x);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = x;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s = red[0];
+    for (int i = 1; i < nw; ++i) s = fmaxf(s, red[i]);
+    red[16] = s;
+  }
+  __syncthreads();
+  return red[16];
+}

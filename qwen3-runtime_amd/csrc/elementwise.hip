@@ -1,0 +1,259 @@
+// Memory-bound ops between the matrix products: embedding gather, residual add
+// + RMSNorm, per-head q/k RMSNorm + rotary encoding + cache write, SwiGLU.
+// All reductions, the norms, the rotation angles and the residual sum are
+// float32; each row's reduction order is fixed, whatever else is in the batch.
+#include "common.h"
+#include <math.h>
+
+// ---------------------------------------------------------------- embedding
+// residual[t, :] = float(table[ids[t], :])            (no scaling of embeddings)
+template <typename TW>
+__global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
+                             float* __restrict__ out, int hidden) {
+  const int t = blockIdx.x;
+  const TW* row = table + (size_t)ids[t] * hidden;
+  float* o = out + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = to_f32<TW>(row[i]);
+}
+
+extern "C" int qrt_embed(const int* ids, const void* table, int table_dtype, float* out,
+                         int num_tokens, int vocab, int hidden, hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && vocab > 0 && hidden > 0, "embed: bad sizes T=%d V=%d H=%d", num_tokens, vocab, hidden);
+  if (num_tokens == 0) return 0;
+  dim3 grid(num_tokens), block(256);
+  if (table_dtype == QRT_F32)
+    embed_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden);
+  else if (table_dtype == QRT_BF16)
+    embed_kernel<bf16_t><<<grid, block, 0, stream>>>(ids, (const bf16_t*)table, out, hidden);
+  else
+    return qrt_fail("embed: unknown table dtype %d", table_dtype);
+  QRT_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ------------------------------------------------------- add + RMSNorm
+// r = rows ? rows[b] : b
+// x = residual[r] (+ delta[r]);  without `rows` the sum is written back.
+// out[b] = x * rsqrt(mean(x^2) + eps) * weight
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                   const float* __restrict__ weight, const int* __restrict__ rows,
+                                   TO* __restrict__ out, int hidden, float eps) {
+  extern __shared__ float xs[];  // hidden floats + 32 for the reduction
+  float* red = xs + hidden;
+  const int b = blockIdx.x;
+  const int r = rows ? rows[b] : b;
+  float* res = residual + (size_t)r * hidden;
+  const TD* del = delta ? delta + (size_t)r * hidden : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float x = res[i];
+    if (del) {
+      x += to_f32<TD>(del[i]);
+      if (!rows) res[i] = x;
+    }
+    xs[i] = x;
+    ss += x * x;
+  }
+  const float total = block_sum(ss, red);
+  const float inv = rsqrtf(total / (float)hidden + eps);
+  TO* o = out + (size_t)b * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_f32<TO>(xs[i] * inv * weight[i]);
+}
+
+extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dtype, const float* weight,
+                               const int* rows, void* out, int out_dtype, int num_out_rows, int hidden,
+                               float eps, hipStream_t stream) {
+  QRT_CHECK(hidden > 0 && num_out_rows >= 0, "add_rmsnorm: bad sizes rows=%d H=%d", num_out_rows, hidden);
+  const size_t smem = ((size_t)hidden + 32) * sizeof(float);
+  QRT_CHECK(smem <= 64 * 1024, "add_rmsnorm: width %d needs %zu bytes of LDS, limit 65536", hidden, smem);
+  if (num_out_rows == 0) return 0;
+  dim3 grid(num_out_rows), block(hidden >= 2048 ? 512 : 256);
+#define LAUNCH(TD, TO)                                                                    \
+  add_rmsnorm_kernel<TD, TO><<<grid, block, smem, stream>>>(residual, (const TD*)delta, weight, rows, \
+                                                            (TO*)out, hidden, eps)
+  if (delta_dtype == QRT_F32 && out_dtype == QRT_F32) LAUNCH(float, float);
+  else if (delta_dtype == QRT_BF16 && out_dtype == QRT_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (delta_dtype == QRT_F32 && out_dtype == QRT_BF16) LAUNCH(float, bf16_t);
+  else if (delta_dtype == QRT_BF16 && out_dtype == QRT_F32) LAUNCH(bf16_t, float);
+  else return qrt_fail("add_rmsnorm: unknown dtypes %d %d", delta_dtype, out_dtype);
+#undef LAUNCH
+  QRT_LAUNCH_CHECK("add_rmsnorm");
+  return 0;
+}
+
+// ------------------------------------------------------------------ SwiGLU
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i],  silu(x) = x / (1 + exp(-x))
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; idx < total; idx += stride) {
+    const size_t t = idx / inter;
+    const int i = (int)(idx - t * inter);
+    const float g = to_f32<T>(gu[t * 2 * inter + i]);
+    const float u = to_f32<T>(gu[t * 2 * inter + inter + i]);
+    out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int qrt_swiglu(const void* gate_up, void* out, int dtype, int num_tokens, int inter,
+                          hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", num_tokens, inter);
+  const size_t total = (size_t)num_tokens * inter;
+  if (total == 0) return 0;
+  const int block = 256;
+  size_t blocks = (total + block - 1) / block;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == QRT_F32)
+    swiglu_kernel<float><<<dim3((unsigned)blocks), block, 0, stream>>>((const float*)gate_up, (float*)out, inter, total);
+  else if (dtype == QRT_BF16)
+    swiglu_kernel<bf16_t><<<dim3((unsigned)blocks), block, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total);
+  else
+    return qrt_fail("swiglu: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("swiglu");
+  return 0;
+}
+
+// ------------------------------- per-head norm + rotary + cache write
+// One wave per (token, head) over the nq query heads, nkv key heads and nkv
+// value heads of a token. Query and key heads: optional RMSNorm over the head
+// (weight [D]), optional NeoX rotation with angle = float(pos) * inv_freq[j]
+// pairing element j with j + D/2. Value heads are copied. Keys and values go to
+// the paged cache (keys [page, head, offset, D], values [page, head, D, offset])
+// and/or to dense outputs; queries go to q_out.
+struct QkArgs {
+  const void* q_in;  long q_stride;   // elements between tokens
+  const void* k_in;  long k_stride;
+  const void* v_in;  long v_stride;
+  const float* q_weight;  // null: no norm
+  const float* k_weight;
+  const float* inv_freq;  // null: no rotation
+  const int* positions;
+  const int* slots;       // null: no cache write
+  void* q_out;            // [T, nq, D] or null
+  void* k_out;            // [T, nkv, D] or null
+  void* v_out;            // [T, nkv, D] or null
+  void* k_cache;
+  void* v_cache;
+  int num_tokens, nq, nkv, nv, head_dim, page_size;
+  float eps;
+};
+
+template <typename T>
+__global__ void qk_norm_rope_store_kernel(QkArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int heads = a.nq + a.nkv + a.nv;
+  const long item = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= (long)a.num_tokens * heads) return;
+  const int t = (int)(item / heads);
+  const int h = (int)(item - (long)t * heads);
+  const int D = a.head_dim, half = D >> 1;
+
+  if (h >= a.nq + a.nkv) {  // value head: copy
+    const int hv = h - a.nq - a.nkv;
+    const T* src = (const T*)a.v_in + (size_t)t * a.v_stride + (size_t)hv * D;
+    if (a.v_out) {
+      T* dst = (T*)a.v_out + ((size_t)t * a.nv + hv) * D;
+      for (int i = lane; i < D; i += 64) dst[i] = src[i];
+    }
+    if (a.slots) {
+      const int slot = a.slots[t];
+      const int page = slot / a.page_size, off = slot - page * a.page_size;
+      T* dst = (T*)a.v_cache + ((size_t)page * a.nv + hv) * D * a.page_size + off;
+      for (int i = lane; i < D; i += 64) dst[(size_t)i * a.page_size] = src[i];
+    }
+    return;
+  }
+
+  const bool is_q = h < a.nq;
+  const int hh = is_q ? h : h - a.nq;
+  const T* src = is_q ? (const T*)a.q_in + (size_t)t * a.q_stride + (size_t)hh * D
+                      : (const T*)a.k_in + (size_t)t * a.k_stride + (size_t)hh * D;
+  const float* w = is_q ? a.q_weight : a.k_weight;
+
+  // each lane owns the pairs (p, p + D/2) for p = lane, lane + 64, ... (D <= 512)
+  float x1[4], x2[4];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int p = lane + 64 * i;
+    x1[i] = x2[i] = 0.f;
+    if (p < half) {
+      x1[i] = to_f32<T>(src[p]);
+      x2[i] = to_f32<T>(src[p + half]);
+      ss += x1[i] * x1[i] + x2[i] * x2[i];
+    }
+  }
+  if (w) {
+    ss = wave_sum(ss);
+    const float inv = rsqrtf(ss / (float)D + a.eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int p = lane + 64 * i;
+      if (p < half) {
+        x1[i] = x1[i] * inv * w[p];
+        x2[i] = x2[i] * inv * w[p + half];
+      }
+    }
+  }
+  if (a.inv_freq) {
+    const float pos = (float)a.positions[t];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int p = lane + 64 * i;
+      if (p < half) {
+        const float ang = pos * a.inv_freq[p];
+        float s, c;
+        sincosf(ang, &s, &c);
+        const float y1 = x1[i] * c - x2[i] * s;
+        const float y2 = x2[i] * c + x1[i] * s;
+        x1[i] = y1;
+        x2[i] = y2;
+      }
+    }
+  }
+  T* dense = nullptr;
+  if (is_q && a.q_out) dense = (T*)a.q_out + ((size_t)t * a.nq + hh) * D;
+  if (!is_q && a.k_out) dense = (T*)a.k_out + ((size_t)t * a.nkv + hh) * D;
+  T* paged = nullptr;
+  if (!is_q && a.slots) {
+    const int slot = a.slots[t];
+    const int page = slot / a.page_size, off = slot - page * a.page_size;
+    paged = (T*)a.k_cache + (((size_t)page * a.nkv + hh) * a.page_size + off) * D;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int p = lane + 64 * i;
+    if (p < half) {
+      const T y1 = from_f32<T>(x1[i]), y2 = from_f32<T>(x2[i]);
+      if (dense) { dense[p] = y1; dense[p + half] = y2; }
+      if (paged) { paged[p] = y1; paged[p + half] = y2; }
+    }
+  }
+}
+
+extern "C" int qrt_qk_norm_rope_store(const QkArgs* args, int dtype, long num_cache_pages, hipStream_t stream) {
+  QkArgs a = *args;
+  QRT_CHECK(a.num_tokens >= 0 && a.nq >= 0 && a.nkv >= 0 && a.nv >= 0, "qk_norm_rope_store: negative size");
+  QRT_CHECK(a.head_dim >= 2 && a.head_dim % 2 == 0 && a.head_dim <= 512,
+            "qk_norm_rope_store: head size %d must be even and at most 512", a.head_dim);
+  QRT_CHECK(a.nq == 0 || a.q_in, "qk_norm_rope_store: query heads without input");
+  QRT_CHECK(a.nkv == 0 || a.k_in, "qk_norm_rope_store: key heads without input");
+  QRT_CHECK(a.nv == 0 || a.v_in, "qk_norm_rope_store: value heads without input");
+  QRT_CHECK(!a.inv_freq || a.positions, "qk_norm_rope_store: rotation without positions");
+  if (a.slots) {
+    QRT_CHECK(a.k_cache && a.v_cache && a.page_size > 0 && num_cache_pages > 0,
+              "qk_norm_rope_store: cache write without cache");
+    QRT_CHECK(a.nkv == a.nv, "qk_norm_rope_store: cache write needs as many key as value heads");
+  }
+  const long items = (long)a.num_tokens * (a.nq + a.nkv + a.nv);
+  if (items == 0) return 0;
+  const int waves = 4;
+  dim3 grid((unsigned)((items + waves - 1) / waves)), block(64 * waves);
+  if (dtype == QRT_F32) qk_norm_rope_store_kernel<float><<<grid, block, 0, stream>>>(a);
+  else if (dtype == QRT_BF16) qk_norm_rope_store_kernel<bf16_t><<<grid, block, 0, stream>>>(a);
+  else return qrt_fail("qk_norm_rope_store: unknown dtype %d", dtype);
+  QRT_LAUNCH_CHECK("qk_norm_rope_store");
+  return 0;
+}

@@ -1,0 +1,18 @@
+// Error reporting shared by all entry points.
+#include "common.h"
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512] = "";
+
+extern "C" const char* qrt_last_error() { return g_error; }
+
+int qrt_fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return -1;
+}
+
+extern "C" int qrt_abi_version() { return 1; }

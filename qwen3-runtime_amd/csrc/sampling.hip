@@ -1,0 +1,272 @@
+// Sampling on the device: one block per row of float32 logits.
+//
+// Chain, in the order the reference runs it (qwen3_runtime/sampling.py:120-135):
+// penalties from per-slot counts, (greedy: first maximal id), temperature,
+// min_p, top_k, top_p, softmax, inverse-CDF draw with a uniform number from a
+// counter-based generator keyed by (seed, draw index). All in float32. top_k
+// and top_p are found by bisection on the value that bounds the kept set, not
+// by sorting; ids that tie with the bound are all kept.
+#include "common.h"
+#include <math.h>
+
+#define SAMPLE_THREADS 1024
+
+// floats ordered as unsigned integers
+__device__ __forceinline__ unsigned f2ord(float f) {
+  const unsigned u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float ord2f(unsigned o) {
+  const unsigned u = (o & 0x80000000u) ? (o & 0x7fffffffu) : ~o;
+  return __uint_as_float(u);
+}
+
+// Philox4x32-10 (Salmon et al. 2011): counter-based, so a draw depends only on
+// (seed, index), never on what else was sampled in the batch.
+__device__ __forceinline__ unsigned mulhi32(unsigned a, unsigned b) { return __umulhi(a, b); }
+__device__ inline float philox_uniform(unsigned long long seed, unsigned long long index) {
+  unsigned c0 = (unsigned)index, c1 = (unsigned)(index >> 32), c2 = 0x51ab1e5u, c3 = 0;
+  unsigned k0 = (unsigned)seed, k1 = (unsigned)(seed >> 32);
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const unsigned h0 = mulhi32(0xD2511F53u, c0), l0 = 0xD2511F53u * c0;
+    const unsigned h1 = mulhi32(0xCD9E8D57u, c2), l1 = 0xCD9E8D57u * c2;
+    const unsigned n0 = h1 ^ c1 ^ k0, n1 = l1, n2 = h0 ^ c3 ^ k1, n3 = l0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return (float)(c0 >> 8) * (1.0f / 16777216.0f);  // [0, 1)
+}
+
+// first maximal index of a row; returns it to every thread
+__device__ int block_argmax(const float* __restrict__ x, int n, float* red, int* redi, float* out_max) {
+  float best = -INFINITY;
+  int besti = 0x7fffffff;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = x[i];
+    if (v > best || (v == best && i < besti)) { best = v; besti = i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(besti, o, 64);
+    if (ov > best || (ov == best && oi < besti)) { best = ov; besti = oi; }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if (lane == 0) { red[wave] = best; redi[wave] = besti; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < nw; ++w)
+      if (red[w] > red[0] || (red[w] == red[0] && redi[w] < redi[0])) { red[0] = red[w]; redi[0] = redi[w]; }
+    if (redi[0] == 0x7fffffff) redi[0] = 0;  // a row of NaNs
+  }
+  __syncthreads();
+  if (out_max) *out_max = red[0];
+  return redi[0];
+}
+
+__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+  __shared__ float red[32];
+  __shared__ int redi[32];
+  const int tok = block_argmax(logits + (size_t)blockIdx.x * vocab, vocab, red, redi, nullptr);
+  if (threadIdx.x == 0) out[blockIdx.x] = tok;
+}
+
+extern "C" int qrt_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+  QRT_CHECK(rows >= 0 && vocab > 0, "argmax: bad sizes");
+  if (rows == 0) return 0;
+  argmax_kernel<<<dim3(rows), dim3(SAMPLE_THREADS), 0, stream>>>(logits, out, vocab);
+  QRT_LAUNCH_CHECK("argmax");
+  return 0;
+}
+
+struct SampleArgs {
+  const float* logits;      // [R, V]
+  float* work;              // [R, V] processed logits (scratch)
+  const int* counts;        // [slots, V] occurrences of each id in prompt + output, or null
+  const int* slot;          // [R] row of counts
+  const float* temperature; // [R]
+  const float* top_p;       // [R]
+  const float* min_p;       // [R]
+  const int* top_k;         // [R]
+  const float* repetition;  // [R]
+  const float* presence;    // [R]
+  const float* frequency;   // [R]
+  const unsigned long long* seed;   // [R]
+  const unsigned long long* draw;   // [R] index of this draw within the request
+  int* out_token;           // [R]
+  float* out_logprob;       // [R]
+  int rows, vocab;
+};
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
+  __shared__ float red[32];
+  __shared__ int redi[32];
+  __shared__ float part[SAMPLE_THREADS];
+  const int r = blockIdx.x, V = a.vocab, tid = threadIdx.x;
+  const float* lg = a.logits + (size_t)r * V;
+  float* x = a.work + (size_t)r * V;
+  const float temp = a.temperature[r];
+
+  // penalties (reference: qwen3_runtime/sampling.py:63-71)
+  const bool pen = a.counts && (a.repetition[r] != 1.0f || a.presence[r] != 0.0f || a.frequency[r] != 0.0f);
+  const int* cnt = pen ? a.counts + (size_t)a.slot[r] * V : nullptr;
+  for (int i = tid; i < V; i += blockDim.x) {
+    float v = lg[i];
+    if (cnt) {
+      const int c = cnt[i];
+      if (c > 0) {
+        v = v > 0.f ? v / a.repetition[r] : v * a.repetition[r];
+        v -= a.presence[r];
+        v -= a.frequency[r] * (float)c;
+      }
+    }
+    if (temp > 0.f) v = v / temp;
+    x[i] = v;
+  }
+  __syncthreads();
+
+  float mx;
+  int best = block_argmax(x, V, red, redi, &mx);
+
+  if (temp <= 0.f) {  // greedy; logprob = log_softmax(processed)[tok]
+    float s = 0.f;
+    for (int i = tid; i < V; i += blockDim.x) s += expf(x[i] - mx);
+    s = block_sum(s, red);
+    if (tid == 0) {
+      a.out_token[r] = best;
+      a.out_logprob[r] = -logf(s);
+    }
+    return;
+  }
+
+  // min_p: drop ids with p < min_p * p_max  <=>  x < max + log(min_p)
+  const float minp = a.min_p[r];
+  if (minp > 0.f) {
+    const float bound = mx + logf(minp);
+    for (int i = tid; i < V; i += blockDim.x)
+      if (x[i] < bound) x[i] = -INFINITY;
+    __syncthreads();
+  }
+
+  // top_k: keep values >= the k-th largest (reference: qwen3_runtime/sampling.py:98-101)
+  int k = a.top_k[r];
+  if (k > 0 && k < V) {
+    unsigned lo = 0u, hi = f2ord(mx);  // largest t with count(x >= t) >= k
+    while (lo < hi) {
+      const unsigned mid = lo + (hi - lo + 1u) / 2u;
+      const float t = ord2f(mid);
+      float c = 0.f;
+      for (int i = tid; i < V; i += blockDim.x) c += (x[i] >= t) ? 1.f : 0.f;
+      c = block_sum(c, red);
+      if (c >= (float)k) lo = mid; else hi = mid - 1u;
+    }
+    const float t = ord2f(lo);
+    for (int i = tid; i < V; i += blockDim.x)
+      if (x[i] < t) x[i] = -INFINITY;
+    __syncthreads();
+  }
+
+  // top_p: keep an id iff the mass of ids strictly above it is <= top_p
+  // (reference: qwen3_runtime/sampling.py:102-109: the first id past the mass stays)
+  const float topp = a.top_p[r];
+  if (topp < 1.0f) {
+    float z = 0.f;
+    for (int i = tid; i < V; i += blockDim.x) z += expf(x[i] - mx);
+    z = block_sum(z, red);
+    unsigned lo = 0u, hi = f2ord(mx);  // smallest t with mass(x > t) <= top_p * z
+    while (lo < hi) {
+      const unsigned mid = lo + (hi - lo) / 2u;
+      const float t = ord2f(mid);
+      float c = 0.f;
+      for (int i = tid; i < V; i += blockDim.x) c += (x[i] > t) ? expf(x[i] - mx) : 0.f;
+      c = block_sum(c, red);
+      if (c <= topp * z) hi = mid; else lo = mid + 1u;
+    }
+    const float t = ord2f(lo);
+    for (int i = tid; i < V; i += blockDim.x)
+      if (x[i] < t) x[i] = -INFINITY;
+    __syncthreads();
+  }
+
+  // softmax + inverse CDF (reference: qwen3_runtime/sampling.py:208-227)
+  const int chunk = (V + blockDim.x - 1) / blockDim.x;
+  const int c0 = min(V, tid * chunk), c1 = min(V, c0 + chunk);
+  float local = 0.f;
+  for (int i = c0; i < c1; ++i) local += expf(x[i] - mx);
+  part[tid] = local;
+  __syncthreads();
+  if (tid == 0) {
+    float run = 0.f;
+    for (int i = 0; i < (int)blockDim.x; ++i) { const float v = part[i]; part[i] = run; run += v; }
+    red[20] = run;
+  }
+  __syncthreads();
+  const float z = red[20];
+  const float u = philox_uniform(a.seed[r], a.draw[r]) * z;
+  if (tid == 0) redi[20] = -1;
+  __syncthreads();
+  // the chunk whose span of the cumulative sum holds u; the last non-empty one if rounding overshoots
+  const float before = part[tid];
+  const float after = (tid + 1 < (int)blockDim.x) ? part[tid + 1] : z;
+  if (local > 0.f && (u < after || after >= z) && u >= before) atomicMax(&redi[20], tid);
+  __syncthreads();
+  int owner = redi[20];
+  if (owner < 0) {  // u fell in no chunk because of rounding: take the last chunk with mass
+    if (local > 0.f) atomicMax(&redi[20], tid);
+    __syncthreads();
+    owner = redi[20];
+  }
+  if (tid == owner) {
+    float run = before;
+    int pick = -1, last = -1;
+    for (int i = c0; i < c1; ++i) {
+      const float pe = expf(x[i] - mx);
+      if (pe > 0.f) {
+        last = i;
+        run += pe;
+        if (run > u) { pick = i; break; }
+      }
+    }
+    if (pick < 0) pick = last;
+    a.out_token[r] = pick;
+    a.out_logprob[r] = logf(fmaxf(expf(x[pick] - mx) / z, 1e-30f));
+  }
+}
+
+extern "C" int qrt_sample(const SampleArgs* args, hipStream_t stream) {
+  SampleArgs a = *args;
+  QRT_CHECK(a.rows >= 0 && a.vocab > 0, "sample: bad sizes");
+  if (a.rows == 0) return 0;
+  sample_kernel<<<dim3(a.rows), dim3(SAMPLE_THREADS), 0, stream>>>(a);
+  QRT_LAUNCH_CHECK("sample");
+  return 0;
+}
+
+// counts[slot[i], token[i]] += 1   (ids a request has seen: prompt and output)
+__global__ void count_tokens_kernel(int* counts, const int* slot, const int* token, int n, int vocab) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) atomicAdd(&counts[(size_t)slot[i] * vocab + token[i]], 1);
+}
+
+extern "C" int qrt_count_tokens(int* counts, const int* slot, const int* token, int n, int vocab, hipStream_t stream) {
+  if (n <= 0) return 0;
+  count_tokens_kernel<<<dim3((n + 255) / 256), dim3(256), 0, stream>>>(counts, slot, token, n, vocab);
+  QRT_LAUNCH_CHECK("count_tokens");
+  return 0;
+}
+
+// logits[row[i], token[i]] += value[i]   (logit bias; reference: qwen3_runtime/sampling.py:35-41)
+__global__ void add_bias_kernel(float* logits, const int* row, const int* token, const float* value, int n, int vocab) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) atomicAdd(&logits[(size_t)row[i] * vocab + token[i]], value[i]);
+}
+
+extern "C" int qrt_add_bias(float* logits, const int* row, const int* token, const float* value, int n, int vocab,
+                            hipStream_t stream) {
+  if (n <= 0) return 0;
+  add_bias_kernel<<<dim3((n + 255) / 256), dim3(256), 0, stream>>>(logits, row, token, value, n, vocab);
+  QRT_LAUNCH_CHECK("add_bias");
+  return 0;
+}

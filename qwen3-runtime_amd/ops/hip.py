@@ -1,0 +1,415 @@
+"""The engine's device ops: thin, checked wrappers over the HIP library.
+
+Each method validates shapes, types and contiguity on the host (a kernel that
+reads past a buffer can take the whole GPU down), then launches on torch's
+current stream through ``ctypes``. There is no other implementation: if the
+library cannot be built or loaded, construction fails. Tensors are torch
+tensors on the GPU; outputs are allocated with torch's caching allocator.
+
+Matrix products: float32 goes to the library's own fused-multiply-add kernel
+(true 32-bit). bfloat16 with few rows, or with float32 output, goes to the
+library's MFMA kernel; bfloat16 with many rows goes to the vendor BLAS through
+``torch.matmul``, as the reference leaves its products to cuBLAS
+(qwen3_runtime/models/qwen3.py:76-77,134-135).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+from ctypes import POINTER, Structure, byref, c_float, c_int, c_long, c_void_p
+
+import numpy as np
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class OpsError(RuntimeError):
+    pass
+
+
+class _QkArgs(Structure):
+    _fields_ = [
+        ("q_in", c_void_p), ("q_stride", c_long),
+        ("k_in", c_void_p), ("k_stride", c_long),
+        ("v_in", c_void_p), ("v_stride", c_long),
+        ("q_weight", c_void_p), ("k_weight", c_void_p), ("inv_freq", c_void_p),
+        ("positions", c_void_p), ("slots", c_void_p),
+        ("q_out", c_void_p), ("k_out", c_void_p), ("v_out", c_void_p),
+        ("k_cache", c_void_p), ("v_cache", c_void_p),
+        ("num_tokens", c_int), ("nq", c_int), ("nkv", c_int), ("nv", c_int),
+        ("head_dim", c_int), ("page_size", c_int), ("eps", c_float),
+    ]
+
+
+class _AttnArgs(Structure):
+    _fields_ = [
+        ("q", c_void_p), ("out", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p),
+        ("positions", c_void_p), ("seq_of_token", c_void_p), ("block_table", c_void_p),
+        ("table_width", c_int), ("num_tokens", c_int), ("nq", c_int), ("nkv", c_int),
+        ("head_dim", c_int), ("page_size", c_int), ("window", c_int), ("scale", c_float),
+    ]
+
+
+class _AttnTileArgs(Structure):
+    _fields_ = [
+        ("q", c_void_p), ("out", c_void_p), ("k_cache", c_void_p), ("v_cache", c_void_p),
+        ("cu_q", c_void_p), ("kv_lens", c_void_p), ("block_table", c_void_p),
+        ("tile_seq", c_void_p), ("tile_row0", c_void_p), ("part_o", c_void_p), ("part_lse", c_void_p),
+        ("table_width", c_int), ("num_tiles", c_int), ("nq", c_int), ("nkv", c_int),
+        ("page_size", c_int), ("window", c_int), ("num_splits", c_int), ("waves", c_int),
+        ("scale_log2", c_float),
+    ]
+
+
+class _SampleArgs(Structure):
+    _fields_ = [
+        ("logits", c_void_p), ("work", c_void_p), ("counts", c_void_p), ("slot", c_void_p),
+        ("temperature", c_void_p), ("top_p", c_void_p), ("min_p", c_void_p), ("top_k", c_void_p),
+        ("repetition", c_void_p), ("presence", c_void_p), ("frequency", c_void_p),
+        ("seed", c_void_p), ("draw", c_void_p), ("out_token", c_void_p), ("out_logprob", c_void_p),
+        ("rows", c_int), ("vocab", c_int),
+    ]
+
+
+def _load(name: str) -> ctypes.CDLL:
+    path = build.build_library(name)
+    try:
+        lib = ctypes.CDLL(str(path))
+    except OSError as exc:
+        raise OpsError(f"cannot load {path}: {exc}") from exc
+    lib.qrt_last_error.restype = ctypes.c_char_p
+    return lib
+
+
+_core: ctypes.CDLL | None = None
+_attn: dict[int, ctypes.CDLL] = {}
+
+
+def core_library() -> ctypes.CDLL:
+    global _core
+    if _core is None:
+        _core = _load("core")
+    return _core
+
+
+def attention_library(head_dim: int) -> ctypes.CDLL:
+    if head_dim not in _attn:
+        _attn[head_dim] = _load(f"attn_bf16_d{head_dim}")
+    return _attn[head_dim]
+
+
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _addr(t: torch.Tensor | None):
+    """Address for a structure field (ctypes takes an int or None there)."""
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> torch.Tensor:
+    if not t.is_cuda:
+        raise OpsError(f"{name} must be on the GPU, it is on {t.device}")
+    if not t.is_contiguous():
+        raise OpsError(f"{name} must be contiguous, strides are {t.stride()} for shape {tuple(t.shape)}")
+    if dtype is not None and t.dtype != dtype:
+        raise OpsError(f"{name} must be {dtype}, it is {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise OpsError(f"{name} must have shape {tuple(shape)}, it has {tuple(t.shape)}")
+    return t
+
+
+class HipOps:
+    # bfloat16 products with more rows than this go to the vendor BLAS
+    blas_min_rows = 128
+
+    def __init__(self):
+        self.lib = core_library()
+
+    def _check(self, lib, code: int) -> None:
+        if code != 0:
+            raise OpsError(lib.qrt_last_error().decode())
+
+    # ---- embedding, norms, activations ---------------------------------------
+    def embed(self, ids, table):
+        _need(ids, "ids", torch.int32)
+        _need(table, "embedding table")
+        t, (v, h) = ids.numel(), table.shape
+        out = torch.empty((t, h), dtype=torch.float32, device=table.device)
+        self._check(self.lib, self.lib.qrt_embed(_ptr(ids), _ptr(table), _CODE[table.dtype], _ptr(out),
+                                                 c_int(t), c_int(v), c_int(h), _stream()))
+        return out
+
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None):
+        t, h = residual.shape
+        _need(residual, "residual", torch.float32)
+        _need(weight, "norm weight", torch.float32, (h,))
+        if delta is not None:
+            _need(delta, "delta", shape=(t, h))
+        n_out = t
+        if rows is not None:
+            _need(rows, "rows", torch.int32)
+            n_out = rows.numel()
+        out = torch.empty((n_out, h), dtype=out_dtype, device=residual.device)
+        self._check(self.lib, self.lib.qrt_add_rmsnorm(
+            _ptr(residual), _ptr(delta), _CODE[delta.dtype] if delta is not None else F32, _ptr(weight),
+            _ptr(rows), _ptr(out), _CODE[out_dtype], c_int(n_out), c_int(h), c_float(eps), _stream()))
+        return out
+
+    def swiglu(self, gate_up):
+        _need(gate_up, "gate_up")
+        t, two_i = gate_up.shape
+        if two_i % 2:
+            raise OpsError(f"gate_up has odd width {two_i}")
+        out = torch.empty((t, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+        self._check(self.lib, self.lib.qrt_swiglu(_ptr(gate_up), _ptr(out), _CODE[gate_up.dtype],
+                                                  c_int(t), c_int(two_i // 2), _stream()))
+        return out
+
+    # ---- matrix products -------------------------------------------------------
+    def linear(self, x, w, out_f32=False):
+        _need(x, "x")
+        _need(w, "weight")
+        m, k = x.shape
+        n, kw = w.shape
+        if k != kw:
+            raise OpsError(f"linear: x is {tuple(x.shape)}, weight is {tuple(w.shape)}")
+        if w.dtype == torch.float32:
+            # true 32-bit product; a float32 weight met by bfloat16 activations keeps its precision
+            xin = x if x.dtype == torch.float32 else x.float()
+            out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+            self._check(self.lib, self.lib.qrt_gemm_f32(_ptr(xin), _ptr(w), _ptr(out), c_int(m), c_int(n),
+                                                        c_int(k), _stream()))
+            return out if (out_f32 or x.dtype == torch.float32) else out.to(x.dtype)
+        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+            raise OpsError(f"linear: no product of {x.dtype} activations with {w.dtype} weights")
+        if m >= self.blas_min_rows and not out_f32:
+            return torch.matmul(x, w.t())
+        out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
+        self._check(self.lib, self.lib.qrt_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), F32 if out_f32 else BF16,
+                                                     c_int(m), c_int(n), c_int(k), _stream()))
+        return out
+
+    # ---- q/k norm, rotation, cache write ----------------------------------------
+    def _qk(self, args: _QkArgs, dtype, num_pages=0):
+        self._check(self.lib, self.lib.qrt_qk_norm_rope_store(byref(args), _CODE[dtype], c_long(num_pages), _stream()))
+
+    def qk_norm_rope_store(self, qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions, cache):
+        t, width = qkv.shape
+        _need(qkv, "qkv", shape=(t, (nq + 2 * nkv) * d))
+        for name, w in (("q_norm", q_w), ("k_norm", k_w)):
+            if w is not None:
+                _need(w, name, torch.float32, (d,))
+        if inv_freq is not None:
+            _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
+            _need(positions, "positions", torch.int32, (t,))
+        q = torch.empty((t, nq * d), dtype=qkv.dtype, device=qkv.device)
+        es = qkv.element_size()
+        a = _QkArgs()
+        a.q_in, a.q_stride = qkv.data_ptr(), width
+        a.k_in, a.k_stride = qkv.data_ptr() + nq * d * es, width
+        a.v_in, a.v_stride = qkv.data_ptr() + (nq + nkv) * d * es, width
+        a.q_weight, a.k_weight, a.inv_freq = _addr(q_w), _addr(k_w), _addr(inv_freq)
+        a.positions = _addr(positions) if inv_freq is not None else None
+        a.q_out = q.data_ptr()
+        a.num_tokens, a.nq, a.nkv, a.nv, a.head_dim, a.eps = t, nq, nkv, nkv, d, eps
+        pages = 0
+        if cache is not None:
+            pages = self._check_cache(cache, nkv, d, qkv.dtype)
+            _need(cache.group.slots, "slots", torch.int32, (t,))
+            a.slots, a.k_cache, a.v_cache = _addr(cache.group.slots), _addr(cache.k), _addr(cache.v)
+            a.page_size = cache.group.page_size
+        else:
+            a.nkv = a.nv = 0  # keys and values go nowhere: only queries are needed
+        self._qk(a, qkv.dtype, pages)
+        return q
+
+    def qk_norm_split(self, qkv, nq, nkv, d, q_w, k_w, eps):
+        t, width = qkv.shape
+        _need(qkv, "qkv", shape=(t, (nq + 2 * nkv) * d))
+        q = torch.empty((t, nq, d), dtype=qkv.dtype, device=qkv.device)
+        k = torch.empty((t, nkv, d), dtype=qkv.dtype, device=qkv.device)
+        v = torch.empty((t, nkv, d), dtype=qkv.dtype, device=qkv.device)
+        es = qkv.element_size()
+        a = _QkArgs()
+        a.q_in, a.q_stride = qkv.data_ptr(), width
+        a.k_in, a.k_stride = qkv.data_ptr() + nq * d * es, width
+        a.v_in, a.v_stride = qkv.data_ptr() + (nq + nkv) * d * es, width
+        a.q_weight, a.k_weight = _addr(q_w), _addr(k_w)
+        a.q_out, a.k_out, a.v_out = q.data_ptr(), k.data_ptr(), v.data_ptr()
+        a.num_tokens, a.nq, a.nkv, a.nv, a.head_dim, a.eps = t, nq, nkv, nkv, d, eps
+        self._qk(a, qkv.dtype)
+        return q, k, v
+
+    def rope_neox(self, q, k, positions, inv_freq):
+        t, nq, d = q.shape
+        nkv = k.shape[1]
+        _need(q, "q")
+        _need(k, "k", q.dtype, (t, nkv, d))
+        _need(inv_freq, "inv_freq", torch.float32, (d // 2,))
+        _need(positions, "positions", torch.int32, (t,))
+        q_out, k_out = torch.empty_like(q), torch.empty_like(k)
+        a = _QkArgs()
+        a.q_in, a.q_stride = q.data_ptr(), nq * d
+        a.k_in, a.k_stride = k.data_ptr(), nkv * d
+        a.inv_freq, a.positions = _addr(inv_freq), _addr(positions)
+        a.q_out, a.k_out = q_out.data_ptr(), k_out.data_ptr()
+        a.num_tokens, a.nq, a.nkv, a.nv, a.head_dim = t, nq, nkv, 0, d
+        self._qk(a, q.dtype)
+        return q_out, k_out
+
+    def kv_store(self, k, v, cache):
+        t, nkv, d = k.shape
+        _need(k, "k")
+        _need(v, "v", k.dtype, (t, nkv, d))
+        pages = self._check_cache(cache, nkv, d, k.dtype)
+        _need(cache.group.slots, "slots", torch.int32, (t,))
+        a = _QkArgs()
+        a.k_in, a.k_stride = k.data_ptr(), nkv * d
+        a.v_in, a.v_stride = v.data_ptr(), nkv * d
+        a.slots, a.k_cache, a.v_cache = _addr(cache.group.slots), _addr(cache.k), _addr(cache.v)
+        a.num_tokens, a.nq, a.nkv, a.nv, a.head_dim = t, 0, nkv, nkv, d
+        a.page_size = cache.group.page_size
+        self._qk(a, k.dtype, pages)
+
+    @staticmethod
+    def _check_cache(cache, nkv, d, dtype) -> int:
+        ps = cache.group.page_size
+        pages = cache.k.shape[0]
+        _need(cache.k, "key cache", dtype, (pages, nkv, ps, d))
+        _need(cache.v, "value cache", dtype, (pages, nkv, d, ps))
+        return pages
+
+    # ---- attention ---------------------------------------------------------------
+    def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window):
+        t = ctx.num_tokens
+        _need(q, "q", shape=(t, nq * d))
+        self._check_cache(cache, nkv, d, q.dtype)
+        table = _need(cache.group.block_table, "block table", torch.int32)
+        if table.shape[0] != ctx.num_seqs:
+            raise OpsError(f"block table has {table.shape[0]} rows for {ctx.num_seqs} sequences")
+        ps = cache.group.page_size
+        need_pages = (ctx.max_kv_len + ps - 1) // ps
+        if table.shape[1] < need_pages:
+            raise OpsError(f"block table is {table.shape[1]} pages wide, the longest sequence needs {need_pages}")
+        out = torch.empty_like(q)
+        if q.dtype == torch.bfloat16 and d % 16 == 0 and ps % 8 == 0:
+            self._attention_mfma(q, out, cache, ctx, nq, nkv, d, scale, window or 0)
+        else:
+            a = _AttnArgs()
+            a.q, a.out, a.k_cache, a.v_cache = q.data_ptr(), out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
+            a.positions = _need(ctx.positions, "positions", torch.int32, (t,)).data_ptr()
+            a.seq_of_token = _need(ctx.seq_of_token, "seq_of_token", torch.int32, (t,)).data_ptr()
+            a.block_table, a.table_width = table.data_ptr(), table.shape[1]
+            a.num_tokens, a.nq, a.nkv, a.head_dim, a.page_size = t, nq, nkv, d, ps
+            a.window, a.scale = window or 0, scale
+            self._check(self.lib, self.lib.qrt_attention_f32(byref(a), _CODE[q.dtype], _stream()))
+        return out
+
+    @staticmethod
+    def plan_tiles(q_lens, group_size: int, waves: int):
+        """Work list of the MFMA attention kernel: (sequence, first row) per tile of 16*waves rows."""
+        rows_per_tile = 16 * waves
+        seqs, row0 = [], []
+        for s, n in enumerate(q_lens):
+            for r in range(0, n * group_size, rows_per_tile):
+                seqs.append(s)
+                row0.append(r)
+        return np.asarray(seqs + row0, dtype=np.int32), len(seqs)
+
+    @staticmethod
+    def choose_splits(num_tiles: int, nkv: int, max_kv: int) -> int:
+        """How many ways to split the keys so that few long sequences still fill the chip."""
+        work = num_tiles * nkv
+        if max_kv <= 512 or work >= 512:
+            return 1
+        return max(1, min((max_kv + 255) // 256, (1024 + work - 1) // work, 64))
+
+    def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window):
+        lib = attention_library(d)
+        g = nq // nkv
+        max_rows = ctx.max_q_len * g
+        waves = 1 if max_rows <= 16 else (2 if max_rows <= 32 else 4)
+        key = ("attn_tiles", g, waves)
+        plan = ctx.scratch.get(key)
+        if plan is None:
+            host, n_tiles = self.plan_tiles(ctx.q_lens_host, g, waves)
+            plan = (torch.from_numpy(host).to(q.device), n_tiles)
+            ctx.scratch[key] = plan
+        tiles, n_tiles = plan
+        splits = ctx.scratch.get("attn_splits") or self.choose_splits(n_tiles, nkv, ctx.max_kv_len)
+        a = _AttnTileArgs()
+        a.q, a.out, a.k_cache, a.v_cache = q.data_ptr(), out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
+        a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
+        a.kv_lens = _need(ctx.kv_lens, "kv_lens", torch.int32, (ctx.num_seqs,)).data_ptr()
+        a.block_table, a.table_width = cache.group.block_table.data_ptr(), cache.group.block_table.shape[1]
+        a.tile_seq = tiles.data_ptr()
+        a.tile_row0 = tiles.data_ptr() + 4 * n_tiles
+        a.num_tiles, a.nq, a.nkv, a.page_size, a.window = n_tiles, nq, nkv, cache.group.page_size, window
+        a.num_splits, a.waves = splits, waves
+        a.scale_log2 = scale * math.log2(math.e)
+        if splits > 1:
+            part_o = torch.empty((ctx.num_tokens * nq * splits, d), dtype=torch.float32, device=q.device)
+            part_lse = torch.empty((ctx.num_tokens * nq * splits,), dtype=torch.float32, device=q.device)
+            a.part_o, a.part_lse = part_o.data_ptr(), part_lse.data_ptr()
+        self._check(lib, lib.qrt_attention_bf16(byref(a), c_int(ctx.num_tokens * nq), _stream()))
+
+    # ---- sampling ------------------------------------------------------------------
+    def argmax(self, logits):
+        _need(logits, "logits", torch.float32)
+        r, v = logits.shape
+        out = torch.empty((r,), dtype=torch.int32, device=logits.device)
+        self._check(self.lib, self.lib.qrt_argmax(_ptr(logits), _ptr(out), c_int(r), c_int(v), _stream()))
+        return out
+
+    def sample(self, logits, params: dict, counts=None):
+        """``params``: device tensors per row: temperature, top_p, min_p, repetition, presence,
+        frequency (float32), top_k, slot (int32), seed, draw (int64). Returns (token, logprob)."""
+        _need(logits, "logits", torch.float32)
+        r, v = logits.shape
+        f32 = ("temperature", "top_p", "min_p", "repetition", "presence", "frequency")
+        for name in f32:
+            _need(params[name], name, torch.float32, (r,))
+        for name in ("top_k", "slot"):
+            _need(params[name], name, torch.int32, (r,))
+        for name in ("seed", "draw"):
+            _need(params[name], name, torch.int64, (r,))
+        if counts is not None:
+            _need(counts, "counts", torch.int32)
+            if counts.shape[1] != v:
+                raise OpsError(f"counts are {counts.shape[1]} wide for a vocabulary of {v}")
+        work = torch.empty_like(logits)
+        tok = torch.empty((r,), dtype=torch.int32, device=logits.device)
+        lp = torch.empty((r,), dtype=torch.float32, device=logits.device)
+        a = _SampleArgs()
+        a.logits, a.work, a.counts = logits.data_ptr(), work.data_ptr(), _addr(counts)
+        for name in f32 + ("top_k", "slot", "seed", "draw"):
+            setattr(a, name, params[name].data_ptr())
+        a.out_token, a.out_logprob, a.rows, a.vocab = tok.data_ptr(), lp.data_ptr(), r, v
+        self._check(self.lib, self.lib.qrt_sample(byref(a), _stream()))
+        return tok, lp
+
+    def count_tokens(self, counts, slots, tokens):
+        _need(counts, "counts", torch.int32)
+        _need(slots, "slots", torch.int32)
+        _need(tokens, "tokens", torch.int32, tuple(slots.shape))
+        self._check(self.lib, self.lib.qrt_count_tokens(_ptr(counts), _ptr(slots), _ptr(tokens),
+                                                        c_int(slots.numel()), c_int(counts.shape[1]), _stream()))
+
+    def add_bias(self, logits, rows, tokens, values):
+        _need(logits, "logits", torch.float32)
+        n = rows.numel()
+        _need(rows, "rows", torch.int32)
+        _need(tokens, "tokens", torch.int32, (n,))
+        _need(values, "values", torch.float32, (n,))
+        self._check(self.lib, self.lib.qrt_add_bias(_ptr(logits), _ptr(rows), _ptr(tokens), _ptr(values),
+                                                    c_int(n), c_int(logits.shape[1]), _stream()))

@@ -1,0 +1,95 @@
+"""The engine on the GPU against the plain implementation, in float32 and bfloat16:
+each request whole; the last 32 tokens one by one; portions of changing size;
+up to four live requests mixed, with so few pages that they are reused."""
+
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import traces
+
+pytestmark = pytest.mark.gpu
+
+ROOT = Path(__file__).resolve().parents[1]
+WORKLOADS = {"tiny_a": [1, 7, 33, 70], "tiny_b": [3, 17, 40, 64, 95]}
+# float32: rounding of a few hundred float32 operations. bfloat16: activations are rounded
+# to 8 bits of mantissa between kernels, logits of these models are of order one.
+TOL = {"float32": dict(atol=5e-5, rtol=5e-5), "bfloat16": dict(atol=3e-2, rtol=3e-2)}
+
+
+def load_gpu(folder, page_size, num_pages, dtype, max_seqs=4, hip_graph=False):
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg = EngineConfig(page_size=page_size, num_pages=num_pages, max_num_seqs=max_seqs, dtype=dtype,
+                       device="cuda:0", hip_graph=hip_graph)
+    return load(folder, cfg)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_b"])
+@pytest.mark.parametrize("cut", ["whole", "tail_one_by_one", "portions", "mixed"])
+def test_cuttings_match_plain(model_folders, tiny_configs, name, cut, dtype):
+    cfg, page = tiny_configs[name]
+    reqs = traces.make_requests(cfg.vocab_size, WORKLOADS[name], seed=5)
+    steps = getattr(traces, cut)(reqs)
+    loaded = load_gpu(model_folders[name], page, traces.peak_tokens(steps) // page, dtype)
+    got = traces.replay(loaded, steps)
+    traces.compare(got, traces.plain_logits(model_folders[name], reqs), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_with_page_reuse(model_folders, tiny_configs, dtype):
+    cfg, page = tiny_configs["tiny_b"]
+    reqs = traces.make_requests(cfg.vocab_size, [40, 64, 95, 17, 33, 80, 130, 2], seed=9)
+    steps = traces.mixed(reqs, seed=3)
+    pages = traces.peak_tokens(steps) // page
+    assert pages < sum(-(-len(t) // page) for t in reqs.values())
+    loaded = load_gpu(model_folders["tiny_b"], page, pages, dtype)
+    got = traces.replay(loaded, steps)
+    traces.compare(got, traces.plain_logits(model_folders["tiny_b"], reqs), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(model_folders, tiny_configs, dtype):
+    """A short prompt, then 400 tokens one by one: crosses many pages and attention key blocks."""
+    cfg, page = tiny_configs["tiny_a"]
+    reqs = traces.make_requests(cfg.vocab_size, [420], seed=2)
+    steps = traces.tail_one_by_one(reqs, tail=400)
+    loaded = load_gpu(model_folders["tiny_a"], page, traces.peak_tokens(steps) // page, dtype)
+    got = traces.replay(loaded, steps)
+    traces.compare(got, traces.plain_logits(model_folders["tiny_a"], reqs), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_folders, tiny_configs, tmp_path, dtype):
+    """bin/trace_run as a user runs it: steps on stdin, files out, 'done' lines."""
+    cfg, page = tiny_configs["tiny_b"]
+    reqs = traces.make_requests(cfg.vocab_size, [19, 45, 70], seed=4)
+    steps = traces.mixed(reqs, seed=1, max_live=3)
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_folders["tiny_b"]),
+         "--dtype", dtype, "--out", str(out), "--max-tokens", str(traces.peak_tokens(steps))],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600,
+    )
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    got, pos = {}, {}
+    for s in steps:
+        n_want = sum(len(e["want"]) for e in s["entries"])
+        if n_want:
+            arr = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(n_want, cfg.vocab_size)
+            row = 0
+            for e in s["entries"]:
+                for w in e["want"]:
+                    got[(e["id"], pos.get(e["id"], 0) + w)] = torch.from_numpy(arr[row].copy())
+                    row += 1
+        for e in s["entries"]:
+            pos[e["id"]] = pos.get(e["id"], 0) + len(e["tokens"])
+    traces.compare(got, traces.plain_logits(model_folders["tiny_b"], reqs), **TOL[dtype])

@@ -1,0 +1,68 @@
+"""The step function, the cache and the ways of cutting, on the CPU.
+
+The engine's ops are replaced by their plain torch versions (the kernels cannot
+run here), so what these tests pin is the host side: packing, block tables,
+slots, page reuse, lengths. Logits must equal the plain implementation's under
+every cutting, in float32.
+"""
+
+import pytest
+import torch
+
+import traces
+from plain.ops_ref import TorchOps
+
+
+def load_cpu(folder, page_size, num_pages, max_seqs=4):
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg = EngineConfig(page_size=page_size, num_pages=num_pages, max_num_seqs=max_seqs, dtype="float32",
+                       device="cpu", hip_graph=False)
+    return load(folder, cfg, ops=TorchOps())
+
+
+WORKLOADS = {"tiny_a": [1, 7, 33, 70], "tiny_b": [3, 17, 40, 64, 95]}
+
+
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_b"])
+@pytest.mark.parametrize("cut", ["whole", "tail_one_by_one", "portions", "mixed"])
+def test_cuttings_match_plain(model_folders, tiny_configs, name, cut):
+    cfg, page = tiny_configs[name]
+    reqs = traces.make_requests(cfg.vocab_size, WORKLOADS[name], seed=5)
+    steps = getattr(traces, cut)(reqs)
+    pages = traces.peak_tokens(steps) // page
+    loaded = load_cpu(model_folders[name], page, pages)
+    got = traces.replay(loaded, steps)
+    traces.compare(got, traces.plain_logits(model_folders[name], reqs), atol=2e-5, rtol=2e-5)
+
+
+def test_pages_are_reused_in_the_mixed_trace(model_folders, tiny_configs):
+    cfg, page = tiny_configs["tiny_b"]
+    reqs = traces.make_requests(cfg.vocab_size, [40, 64, 95, 17, 33, 80], seed=9)
+    steps = traces.mixed(reqs, seed=3)
+    pages = traces.peak_tokens(steps) // page
+    total_needed = sum(-(-len(t) // page) for t in reqs.values())
+    assert pages < total_needed  # so some page must serve two requests
+    loaded = load_cpu(model_folders["tiny_b"], page, pages)
+    got = traces.replay(loaded, steps)
+    traces.compare(got, traces.plain_logits(model_folders["tiny_b"], reqs), atol=2e-5, rtol=2e-5)
+
+
+def test_step_refuses_bad_entries(model_folders, tiny_configs):
+    from qwen3_runtime_amd.cache import CacheFull
+    from qwen3_runtime_amd.engine.batch import StepEntry
+
+    cfg, page = tiny_configs["tiny_a"]
+    loaded = load_cpu(model_folders["tiny_a"], page, 2)
+    loaded.cache.admit("a")
+    with pytest.raises(ValueError, match="twice"):
+        loaded.runner.step([StepEntry("a", [1]), StepEntry("a", [2])])
+    with pytest.raises(ValueError, match="outside"):
+        loaded.runner.step([StepEntry("a", [cfg.vocab_size])])
+    with pytest.raises(ValueError, match="wants row"):
+        loaded.runner.step([StepEntry("a", [1, 2], want=[2])])
+    with pytest.raises(CacheFull):
+        loaded.runner.step([StepEntry("a", list(range(3 * page)))])
+    assert loaded.cache.length("a") == 0
+    loaded.cache.check()

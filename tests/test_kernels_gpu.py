@@ -1,0 +1,273 @@
+"""Each HIP kernel alone against its plain torch reference (tests/plain/ops_ref.py),
+at sizes other than the engine's: odd widths, head sizes in steps of 16, group
+sizes that do not divide a tile, pages of 8 to 64 tokens."""
+
+import math
+
+import pytest
+import torch
+
+from plain import ops_ref as R
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    return HipOps()
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def close(got, want, atol, rtol):
+    torch.testing.assert_close(got.float().cpu(), want.float().cpu(), atol=atol, rtol=rtol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("v,h,t", [(300, 100, 7), (64, 2560, 3)])
+def test_embed(ops, dtype, v, h, t):
+    table = rnd(v, h, dtype=dtype)
+    ids = torch.randint(0, v, (t,), dtype=torch.int32, device=DEV)
+    close(ops.embed(ids, table), R.embed(ids, table), 0, 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("t,h,eps", [(5, 96, 1e-5), (3, 2560, 1e-6), (9, 1000, 1e-6)])
+def test_add_rmsnorm(ops, dtype, t, h, eps):
+    res = rnd(t, h, seed=1)
+    delta = rnd(t, h, dtype=dtype, seed=2)
+    w = (1 + 0.1 * rnd(h, seed=3)).contiguous()
+    want_res = res.clone()
+    want = R.add_rmsnorm(want_res, delta, w, eps, dtype)
+    got_res = res.clone()
+    got = ops.add_rmsnorm(got_res, delta, w, eps, dtype)
+    close(got_res, want_res, 0, 0)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    close(got, want, tol, tol)
+    # no delta; rows subset leaves the residual alone
+    rows = torch.tensor([t - 1, 0], dtype=torch.int32, device=DEV)
+    got_res = res.clone()
+    got = ops.add_rmsnorm(got_res, delta, w, eps, dtype, rows)
+    close(got_res, res, 0, 0)
+    close(got, R.add_rmsnorm(res.clone(), delta, w, eps, dtype, rows), tol, tol)
+    close(ops.add_rmsnorm(res.clone(), None, w, eps, dtype), R.add_rmsnorm(res.clone(), None, w, eps, dtype), tol, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(ops, dtype):
+    gu = rnd(11, 2 * 272, dtype=dtype, scale=3.0)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    close(ops.swiglu(gu), R.swiglu(gu), tol, tol)
+    zero_gate = gu.clone()
+    zero_gate[:, :272] = 0
+    assert ops.swiglu(zero_gate).abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (7, 272, 96), (33, 100, 50), (130, 384, 192), (65, 1000, 2560)])
+def test_gemm_f32(ops, m, n, k):
+    x, w = rnd(m, k, seed=1), rnd(n, k, seed=2, scale=0.05)
+    want = (x.double() @ w.double().T).float()
+    close(ops.linear(x, w), want, 1e-4, 1e-4)
+
+
+def test_gemm_f32_rows_do_not_depend_on_batch(ops):
+    x, w = rnd(70, 200, seed=1), rnd(150, 200, seed=2)
+    whole = ops.linear(x, w)
+    alone = ops.linear(x[40:41].contiguous(), w)
+    assert torch.equal(whole[40:41], alone)
+
+
+@pytest.mark.parametrize("out_f32", [False, True])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (8, 272, 96), (17, 100, 48), (40, 384, 272), (100, 1000, 2560),
+                                   (3, 50, 20)])
+def test_gemm_bf16(ops, m, n, k, out_f32):
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    want = x.double() @ w.double().T
+    got = ops.linear(x, w, out_f32=out_f32)
+    assert got.dtype == (torch.float32 if out_f32 else torch.bfloat16)
+    if out_f32:
+        close(got, want, 1e-3, 1e-3)
+    else:
+        close(got, want, 2e-2, 2e-2)
+
+
+def test_gemm_bf16_large_uses_blas_and_agrees(ops):
+    x, w = rnd(300, 512, dtype=torch.bfloat16, seed=1), rnd(640, 512, dtype=torch.bfloat16, seed=2, scale=0.05)
+    close(ops.linear(x, w), x.double() @ w.double().T, 3e-2, 3e-2)
+    close(ops.linear(x, w, out_f32=True), x.double() @ w.double().T, 1e-3, 1e-3)
+
+
+def test_float32_weight_with_bfloat16_activations_stays_float32(ops):
+    x, w = rnd(5, 64, dtype=torch.bfloat16), rnd(48, 64, scale=0.1)
+    close(ops.linear(x, w, out_f32=True), x.double() @ w.double().T, 1e-5, 1e-5)
+
+
+def make_cache(pages, nkv, ps, d, dtype):
+    from qwen3_runtime_amd.parts.base import CacheView, GroupView
+    from qwen3_runtime_amd.parts.plan import CacheSpec
+
+    k = torch.zeros(pages, nkv, ps, d, dtype=dtype, device=DEV)
+    v = torch.zeros(pages, nkv, d, ps, dtype=dtype, device=DEV)
+    view = CacheView(CacheSpec("paged_kv", heads=nkv, head_dim=d), group=GroupView(ps, None, None, None), k=k, v=v)
+    return view
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,d,ps,theta", [(4, 2, 16, 16, 1e4), (6, 2, 32, 8, 1e6), (3, 1, 80, 4, 5e5),
+                                               (8, 8, 128, 32, 1e6), (2, 1, 256, 16, 1e4)])
+def test_qk_norm_rope_store(ops, dtype, nq, nkv, d, ps, theta):
+    t, pages = 13, 12
+    qkv = rnd(t, (nq + 2 * nkv) * d, dtype=dtype)
+    qw, kw = 1 + 0.1 * rnd(d, seed=5), 1 + 0.1 * rnd(d, seed=6)
+    inv = (1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    pos = torch.tensor([0, 1, 2, 3, 500, 501, 7, 8, 9, 4000, 4001, 30000, 5], dtype=torch.int32, device=DEV)
+    slots = torch.randperm(pages * ps)[:t].to(torch.int32).to(DEV)
+    cache = make_cache(pages, nkv, ps, d, dtype)
+    cache.group.slots = slots
+    want_cache = make_cache(pages, nkv, ps, d, dtype)
+    want = R.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, pos, want_cache.k, want_cache.v, slots, ps)
+    got = ops.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, pos, cache)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    close(got, want, tol, tol)
+    close(cache.k, want_cache.k, tol, tol)
+    close(cache.v, want_cache.v, 0, 0)
+    # no norm, no rotation: a copy
+    got = ops.qk_norm_rope_store(qkv, nq, nkv, d, None, None, 0.0, None, pos, None)
+    close(got, qkv[:, : nq * d], 0, 0)
+    # unfused pieces agree with the fused pass
+    q, k, v = ops.qk_norm_split(qkv, nq, nkv, d, qw, kw, 1e-6)
+    q, k = ops.rope_neox(q, k, pos, inv)
+    cache2 = make_cache(pages, nkv, ps, d, dtype)
+    cache2.group.slots = slots
+    ops.kv_store(k, v, cache2)
+    close(q.reshape(t, -1), want, tol, tol)
+    close(cache2.k, want_cache.k, tol, tol)
+    close(cache2.v, want_cache.v, 0, 0)
+
+
+def build_attention_case(seqs, nq, nkv, d, ps, dtype, seed=0, window=None, shuffle=True, spare_pages=3):
+    """seqs: list of (q_len, kv_len). Returns q, cache view with filled pages, ctx."""
+    from qwen3_runtime_amd.parts.base import StepContext
+
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum((kv + ps - 1) // ps for _, kv in seqs) + spare_pages
+    order = torch.randperm(total_pages, generator=g) if shuffle else torch.arange(total_pages)
+    width = max((kv + ps - 1) // ps for _, kv in seqs)
+    table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    cache = make_cache(total_pages, nkv, ps, d, dtype)
+    # stale content everywhere: a kernel that reads past kv_len or a foreign page shows
+    cache.k.copy_((torch.randn(cache.k.shape, generator=g) * 3).to(dtype))
+    cache.v.copy_((torch.randn(cache.v.shape, generator=g) * 3).to(dtype))
+    nxt = 0
+    for s, (_, kv) in enumerate(seqs):
+        n = (kv + ps - 1) // ps
+        table[s, :n] = order[nxt: nxt + n].to(torch.int32)
+        nxt += n
+    t = sum(q for q, _ in seqs)
+    q = (torch.randn(t, nq * d, generator=g)).to(dtype).to(DEV)
+    cu = [0]
+    positions, seq_of = [], []
+    for s, (ql, kv) in enumerate(seqs):
+        cu.append(cu[-1] + ql)
+        positions += list(range(kv - ql, kv))
+        seq_of += [s] * ql
+    cache.group.block_table = table.to(DEV)
+    cache.group.window = window
+    dev_i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    ctx = StepContext(
+        ops=None, dtype=dtype, device=torch.device(DEV), num_tokens=t, num_seqs=len(seqs),
+        positions=dev_i32(positions), cu_q=dev_i32(cu), kv_lens=dev_i32([kv for _, kv in seqs]),
+        seq_of_token=dev_i32(seq_of), state_slots=dev_i32([0] * len(seqs)), first_span=dev_i32([0] * len(seqs)),
+        q_lens_host=[ql for ql, _ in seqs], kv_lens_host=[kv for _, kv in seqs],
+        max_q_len=max(ql for ql, _ in seqs), max_kv_len=max(kv for _, kv in seqs), groups=[cache.group],
+    )
+    return q, cache, ctx
+
+
+ATTN_CASES = [
+    # (seqs, nq, nkv, d, page)
+    ([(1, 1)], 4, 2, 16, 16),
+    ([(7, 7), (1, 40), (33, 33)], 4, 2, 16, 16),
+    ([(5, 37), (1, 17), (2, 95), (24, 24)], 6, 2, 32, 8),
+    ([(1, 300), (1, 17), (1, 64), (1, 65)], 6, 2, 32, 8),
+    ([(70, 70)], 5, 1, 48, 24),
+    ([(3, 130), (64, 64)], 8, 2, 64, 64),
+    ([(40, 200), (1, 1000)], 32, 8, 128, 16),
+    ([(9, 50)], 3, 3, 80, 16),
+    ([(1, 700)], 34, 2, 16, 32),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seqs,nq,nkv,d,ps", ATTN_CASES)
+def test_paged_attention(ops, dtype, seqs, nq, nkv, d, ps):
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, dtype)
+    scale = 1.0 / math.sqrt(d)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, scale)
+    got = ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, None)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    close(got, want, tol, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 5, 32, 100])
+def test_paged_attention_window(ops, dtype, window):
+    seqs, nq, nkv, d, ps = [(6, 90), (1, 41), (50, 50)], 4, 2, 32, 8
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, dtype, window=window)
+    # pages wholly below the window of the first query are gone
+    table = cache.group.block_table.clone()
+    for s, (ql, kv) in enumerate(seqs):
+        first_needed = kv - ql - window + 1
+        for p in range(table.shape[1]):
+            if (p + 1) * ps <= first_needed:
+                table[s, p] = -1
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, 0.25, window)
+    cache.group.block_table = table
+    got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 0.25, window)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    close(got, want, tol, tol)
+
+
+def test_paged_attention_splits_agree(ops):
+    """Long single sequences split over many blocks; empty splits must not leak."""
+    seqs, nq, nkv, d, ps = [(1, 2100), (1, 40), (3, 900)], 8, 2, 64, 16
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, 0.125)
+    for splits in (1, 2, 7, 40):
+        ctx.scratch["attn_splits"] = splits
+        got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 0.125, None)
+        close(got, want, 2e-2, 2e-2)
+
+
+def test_attention_far_key_stands_out(ops):
+    """One early key is made to dominate; the context must equal its value."""
+    for dtype in (torch.float32, torch.bfloat16):
+        seqs, nq, nkv, d, ps = [(1, 777)], 4, 2, 32, 16
+        q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, dtype)
+        table = cache.group.block_table[0]
+        far = 3
+        page, off = int(table[far // ps]), far % ps
+        cache.k[page, :, off, :] = 0
+        cache.k[page, :, off, 0] = 40.0
+        q[:] = 0
+        q[:, ::d] = 40.0  # element 0 of every head
+        got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 1.0, None)
+        want = cache.v[page, :, :, off].repeat_interleave(nq // nkv, dim=0).reshape(1, -1)
+        close(got, want, 1e-2, 1e-2)
+
+
+def test_argmax_first_maximum(ops):
+    x = torch.tensor([[1.0, 3.0, 3.0, 2.0], [0.0, 0.0, 0.0, 0.0], [3.0, -1.0, 2.5, 3.0]], device=DEV)
+    assert ops.argmax(x).tolist() == [1, 0, 0]
+    big = rnd(5, 151936)
+    assert ops.argmax(big).tolist() == torch.argmax(big, dim=-1).tolist()

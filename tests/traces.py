@@ -1,0 +1,171 @@
+"""Ways of cutting the same requests into steps, and a driver that replays them.
+
+A trace is a list of steps in trace_run's format. ``replay`` drives the
+engine's own step function and cache manager in-process and returns the logits
+by (request, position); ``plain_logits`` gives the same from the plain
+implementation, whole sequences at once.
+"""
+
+from __future__ import annotations
+
+import random
+
+import torch
+
+
+def whole(requests):
+    """Each request alone, in one step, logits everywhere."""
+    steps = []
+    for i, (rid, toks) in enumerate(requests.items()):
+        steps.append({"step": i, "entries": [{"id": rid, "tokens": toks, "want": list(range(len(toks)))}],
+                      "end": [rid]})
+    return steps
+
+
+def tail_one_by_one(requests, tail=32):
+    """Most of the request in one step, the last ``tail`` tokens one by one."""
+    steps = []
+    for rid, toks in requests.items():
+        head = max(1, len(toks) - tail)
+        steps.append({"entries": [{"id": rid, "tokens": toks[:head], "want": list(range(head))}], "end": []})
+        for p in range(head, len(toks)):
+            steps.append({"entries": [{"id": rid, "tokens": toks[p: p + 1], "want": [0]}], "end": []})
+        steps[-1]["end"] = [rid]
+    return _number(steps)
+
+
+def portions(requests, sizes=(24, 7, 2, 16, 3, 2, 31, 5)):
+    """Portions of changing size, down to two tokens."""
+    steps = []
+    for rid, toks in requests.items():
+        p, i = 0, 0
+        while p < len(toks):
+            n = min(sizes[i % len(sizes)], len(toks) - p)
+            steps.append({"entries": [{"id": rid, "tokens": toks[p: p + n], "want": list(range(n))}], "end": []})
+            p += n
+            i += 1
+        steps[-1]["end"] = [rid]
+    return _number(steps)
+
+
+def mixed(requests, seed=0, max_live=4, decode_tail=8):
+    """Up to ``max_live`` requests at once: portions of some beside single tokens of others.
+
+    Each request is fed in portions of random size until ``decode_tail`` tokens
+    remain, which come one per step. A finished request ends at once and the
+    next one starts, so its pages are taken by later tokens of other requests.
+    """
+    rng = random.Random(seed)
+    waiting = list(requests.items())
+    live: dict[str, int] = {}
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid, _ = waiting.pop(0)
+            live[rid] = 0
+        entries, ended = [], []
+        for rid in list(live):
+            toks = requests[rid]
+            p = live[rid]
+            left = len(toks) - p
+            if rng.random() < 0.2 and len(live) > 1 and entries:
+                continue  # a request may sit a step out
+            if left <= decode_tail:
+                n = 1
+            else:
+                n = min(left - decode_tail, rng.choice((2, 3, 5, 9, 17, 30)))
+            entries.append({"id": rid, "tokens": toks[p: p + n], "want": list(range(n))})
+            live[rid] = p + n
+            if p + n == len(toks):
+                ended.append(rid)
+        for rid in ended:
+            del live[rid]
+        if entries:
+            steps.append({"entries": entries, "end": ended})
+    return _number(steps)
+
+
+def _number(steps):
+    for i, s in enumerate(steps):
+        s["step"] = i
+    return steps
+
+
+def peak_tokens(steps, unit=64):
+    """Most tokens live requests hold at any time, each rounded up to ``unit``."""
+    held: dict[str, int] = {}
+    peak = 0
+    for s in steps:
+        for e in s["entries"]:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        peak = max(peak, sum(-(-n // unit) * unit for n in held.values()))
+        for rid in s["end"]:
+            held.pop(rid, None)
+    return peak
+
+
+def replay(loaded, steps, check_cache=True):
+    """Run the steps through ``loaded.runner``; returns {(request, position): logits row}."""
+    from qwen3_runtime_amd.engine.batch import StepEntry
+
+    runner, cache = loaded.runner, loaded.cache
+    pos: dict[str, int] = {}
+    out = {}
+    for s in steps:
+        entries = []
+        for e in s["entries"]:
+            if not cache.has(e["id"]):
+                cache.admit(e["id"])
+                pos[e["id"]] = 0
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+        logits = runner.step(entries)
+        if logits is not None:
+            logits = logits.float().cpu()
+            row = 0
+            for e in s["entries"]:
+                for w in e["want"]:
+                    out[(e["id"], pos[e["id"]] + w)] = logits[row]
+                    row += 1
+            assert row == logits.shape[0]
+        for e in s["entries"]:
+            pos[e["id"]] += len(e["tokens"])
+        for rid in s["end"]:
+            cache.release(rid)
+        if check_cache:
+            cache.check()
+    assert not cache.live_requests()
+    return out
+
+
+def plain_logits(folder, requests):
+    from plain import qwen3_plain as P
+
+    cfg, w = P.read_model(folder)
+    out = {}
+    for rid, toks in requests.items():
+        logits = P.forward(cfg, w, toks)
+        for p in range(len(toks)):
+            out[(rid, p)] = logits[p].float()
+    return out
+
+
+def make_requests(vocab, lengths, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return {f"r{i}": torch.randint(0, vocab, (n,), generator=g).tolist() for i, n in enumerate(lengths)}
+
+
+def compare(got, want, atol, rtol):
+    assert set(got) == set(want), f"{len(set(want) - set(got))} positions are missing"
+    worst, where, first = 0.0, None, None
+    for key in sorted(want):
+        err = (got[key].double() - want[key].double()).abs()
+        bound = atol + rtol * want[key].double().abs()
+        excess = float((err - bound).max())
+        if excess > 0 and first is None:
+            first = (key, float(err.max()))
+        if excess > worst:
+            worst, where = excess, (key, float(err.max()))
+    assert where is None, (
+        f"first mismatch at (request, position) {first[0]} with max abs error {first[1]:.3e}; "
+        f"worst at {where[0]} with {where[1]:.3e}"
+    )
