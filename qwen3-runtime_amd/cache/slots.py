@@ -26,12 +26,19 @@ class StateSlots:
         self._free = list(range(self.num_slots - 1, -1, -1))
         self._slot_of: dict[Hashable, int] = {}
         self.tensors: dict[str, torch.Tensor] = {}
+        self._survives_restart: set[str] = set()
 
-    def add_tensor(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+    def add_tensor(self, name: str, shape: Sequence[int], dtype: torch.dtype,
+                   survives_restart: bool = False) -> torch.Tensor:
+        """One row of ``shape`` per slot. State that follows the tokens in the cache (a mixer's
+        recurrence) is zeroed when its request starts over; state that follows the request
+        (the sampler's draw counter) survives that: pass ``survives_restart``."""
         if name in self.tensors:
             raise ValueError(f"state tensor {name!r} is registered twice")
         t = torch.zeros((self.num_slots, *shape), dtype=dtype, device=self.device)
         self.tensors[name] = t
+        if survives_restart:
+            self._survives_restart.add(name)
         return t
 
     @property
@@ -51,14 +58,16 @@ class StateSlots:
             raise CacheFull("no free state slot")
         slot = self._free.pop()
         self._slot_of[holder] = slot
-        self.reset(holder)
+        for t in self.tensors.values():
+            t[slot].zero_()
         return slot
 
     def reset(self, holder: Hashable) -> None:
-        """Zero the holder's rows: a new request, or one that starts over."""
+        """The holder starts over from position 0: zero the state that followed its tokens."""
         slot = self._slot_of[holder]
-        for t in self.tensors.values():
-            t[slot].zero_()
+        for name, t in self.tensors.items():
+            if name not in self._survives_restart:
+                t[slot].zero_()
 
     def give(self, holder: Hashable) -> None:
         if holder not in self._slot_of:

@@ -81,20 +81,18 @@ extern "C" int qrt_argmax(const float* logits, int* out, int rows, int vocab, hi
   return 0;
 }
 
+// Per-request options live in the request's state slot, written once when the
+// request is admitted: fparams[slot] = {temperature, top_p, min_p, repetition,
+// presence, frequency, -, -}; iparams[slot] = {top_k, -}; seeds[slot] = {seed,
+// index of the next draw}. The kernel advances the draw index itself.
 struct SampleArgs {
   const float* logits;      // [R, V]
-  float* work;              // [R, V] processed logits (scratch)
+  float* work;              // [R, V] processed logits (scratch, returned to the caller)
   const int* counts;        // [slots, V] occurrences of each id in prompt + output, or null
-  const int* slot;          // [R] row of counts
-  const float* temperature; // [R]
-  const float* top_p;       // [R]
-  const float* min_p;       // [R]
-  const int* top_k;         // [R]
-  const float* repetition;  // [R]
-  const float* presence;    // [R]
-  const float* frequency;   // [R]
-  const unsigned long long* seed;   // [R]
-  const unsigned long long* draw;   // [R] index of this draw within the request
+  const int* slot;          // [R] state slot of each row
+  const float* fparams;     // [slots, 8]
+  const int* iparams;       // [slots, 2]
+  unsigned long long* seeds;  // [slots, 2]
   int* out_token;           // [R]
   float* out_logprob;       // [R]
   int rows, vocab;
@@ -107,19 +105,21 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   const int r = blockIdx.x, V = a.vocab, tid = threadIdx.x;
   const float* lg = a.logits + (size_t)r * V;
   float* x = a.work + (size_t)r * V;
-  const float temp = a.temperature[r];
+  const int sl = a.slot[r];
+  const float* fp = a.fparams + (size_t)sl * 8;
+  const float temp = fp[0], topp = fp[1], minp = fp[2], rep = fp[3], pres = fp[4], freq = fp[5];
 
   // penalties (reference: qwen3_runtime/sampling.py:63-71)
-  const bool pen = a.counts && (a.repetition[r] != 1.0f || a.presence[r] != 0.0f || a.frequency[r] != 0.0f);
-  const int* cnt = pen ? a.counts + (size_t)a.slot[r] * V : nullptr;
+  const bool pen = a.counts && (rep != 1.0f || pres != 0.0f || freq != 0.0f);
+  const int* cnt = pen ? a.counts + (size_t)sl * V : nullptr;
   for (int i = tid; i < V; i += blockDim.x) {
     float v = lg[i];
     if (cnt) {
       const int c = cnt[i];
       if (c > 0) {
-        v = v > 0.f ? v / a.repetition[r] : v * a.repetition[r];
-        v -= a.presence[r];
-        v -= a.frequency[r] * (float)c;
+        v = v > 0.f ? v / rep : v * rep;
+        v -= pres;
+        v -= freq * (float)c;
       }
     }
     if (temp > 0.f) v = v / temp;
@@ -142,7 +142,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   }
 
   // min_p: drop ids with p < min_p * p_max  <=>  x < max + log(min_p)
-  const float minp = a.min_p[r];
   if (minp > 0.f) {
     const float bound = mx + logf(minp);
     for (int i = tid; i < V; i += blockDim.x)
@@ -151,9 +150,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   }
 
   // top_k: keep values >= the k-th largest (reference: qwen3_runtime/sampling.py:98-101)
-  int k = a.top_k[r];
+  const int k = a.iparams[(size_t)sl * 2];
   if (k > 0 && k < V) {
-    unsigned lo = 0u, hi = f2ord(mx);  // largest t with count(x >= t) >= k
+    unsigned lo = f2ord(-INFINITY), hi = f2ord(mx);  // largest t with count(x >= t) >= k
     while (lo < hi) {
       const unsigned mid = lo + (hi - lo + 1u) / 2u;
       const float t = ord2f(mid);
@@ -170,12 +169,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
 
   // top_p: keep an id iff the mass of ids strictly above it is <= top_p
   // (reference: qwen3_runtime/sampling.py:102-109: the first id past the mass stays)
-  const float topp = a.top_p[r];
   if (topp < 1.0f) {
     float z = 0.f;
     for (int i = tid; i < V; i += blockDim.x) z += expf(x[i] - mx);
     z = block_sum(z, red);
-    unsigned lo = 0u, hi = f2ord(mx);  // smallest t with mass(x > t) <= top_p * z
+    unsigned lo = f2ord(-INFINITY), hi = f2ord(mx);  // smallest t with mass(x > t) <= top_p * z
     while (lo < hi) {
       const unsigned mid = lo + (hi - lo) / 2u;
       const float t = ord2f(mid);
@@ -204,7 +202,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   }
   __syncthreads();
   const float z = red[20];
-  const float u = philox_uniform(a.seed[r], a.draw[r]) * z;
+  const unsigned long long seed = a.seeds[(size_t)sl * 2], draw = a.seeds[(size_t)sl * 2 + 1];
+  const float u = philox_uniform(seed, draw) * z;
   if (tid == 0) redi[20] = -1;
   __syncthreads();
   // the chunk whose span of the cumulative sum holds u; the last non-empty one if rounding overshoots
@@ -232,6 +231,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
     if (pick < 0) pick = last;
     a.out_token[r] = pick;
     a.out_logprob[r] = logf(fmaxf(expf(x[pick] - mx) / z, 1e-30f));
+    a.seeds[(size_t)sl * 2 + 1] = draw + 1;
   }
 }
 

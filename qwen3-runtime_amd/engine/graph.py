@@ -1,0 +1,106 @@
+"""Pure-decode steps replayed from captured HIP graphs.
+
+A graph is captured per (batch size, bucket of the longest context). Its
+kernels read the step's arrays (token ids, positions, lengths, block tables,
+slots) from one static device buffer; a replay fills that buffer with one copy
+and launches the whole step at once, which removes the per-kernel launch cost
+that otherwise exceeds the time the kernels need at small batch
+(reference, same idea per batch size: qwen3_runtime/engine/cuda_graph.py:82-104,152-188).
+The bucket fixes what a capture freezes: the width of the block table and the
+number of key splits of the attention kernel. Nothing that clears memory with
+a memset node is recorded.
+"""
+
+from __future__ import annotations
+
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from .batch import StepEntry, pack_step
+
+MIN_BUCKET = 512
+
+
+class DecodeGraph:
+    @staticmethod
+    def key_for(batch: int, max_kv: int, all_want: bool):
+        if not all_want:
+            return None
+        bucket = MIN_BUCKET
+        while bucket < max_kv:
+            bucket *= 2
+        return (batch, bucket)
+
+    def __init__(self, runner, key):
+        self.runner = runner
+        self.batch, self.bucket = key
+        cache = runner.cache
+        self.width = max(1, -(-self.bucket // cache.page_size))
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self.logits = None
+        self.layout: list[tuple[str, int, tuple]] | None = None
+        self.host = self.dev = None
+        self.copied = torch.cuda.Event()
+        self.ctx = None
+        self.runs = 0
+
+    def _fill(self, entries: Sequence[StepEntry]):
+        runner = self.runner
+        packed = pack_step(entries, runner.cache, runner.vocab_size, table_width=self.width)
+        if self.layout is None:
+            off, layout = 0, []
+            for name, a in packed.arrays.items():
+                layout.append((name, off, a.shape))
+                off += (a.size + 3) // 4 * 4
+            self.layout, total = layout, max(off, 4)
+            self.host = torch.empty(total, dtype=torch.int32, pin_memory=True)
+            self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        else:
+            self.copied.synchronize()  # the previous copy has left the host buffer
+        host = self.host.numpy()
+        for name, off, shape in self.layout:
+            a = packed.arrays[name]
+            if a.shape != shape:
+                raise AssertionError(f"decode graph: array {name} changed shape {shape} -> {a.shape}")
+            host[off: off + a.size] = a.reshape(-1)
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+        return packed
+
+    def _views(self):
+        return {name: self.dev[off: off + int(np.prod(shape))].view(shape) for name, off, shape in self.layout}
+
+    def run(self, entries: Sequence[StepEntry]):
+        runner = self.runner
+        packed = self._fill(entries)
+        if self.graph is None:
+            if self.ctx is None:
+                self.views_dev = self._views()
+                packed.kv_lens = [self.bucket] * self.batch  # launch shapes are those of the bucket
+                self.ctx = runner._context(packed, self.views_dev)
+                self.ctx.scratch["attn_splits"] = runner.ops.choose_splits(
+                    self.batch, self._min_kv_heads(), self.bucket)
+                self.cache_views = [
+                    None if st.cache is None else runner.cache.view(st.cache, self.ctx.groups, st.writes_cache)
+                    for st in runner.model.plan.order
+                ]
+            dev = self.views_dev
+            self.runs += 1
+            with torch.inference_mode():
+                if self.runs < 2:
+                    # the first call at this size runs eagerly: it fills the attention work list
+                    # and warms the allocator; the capture happens on the second call
+                    return runner.model.forward(self.ctx, dev["ids"], self.cache_views, dev["rows"])
+                graph = torch.cuda.CUDAGraph()
+                torch.cuda.synchronize(runner.device)
+                with torch.cuda.graph(graph):
+                    self.logits = runner.model.forward(self.ctx, dev["ids"], self.cache_views, dev["rows"])
+                self.graph = graph
+        self.graph.replay()
+        return self.logits
+
+    def _min_kv_heads(self) -> int:
+        heads = [s.heads for s in self.runner.model.plan.caches if s.kind == "paged_kv"]
+        return min(heads) if heads else 1

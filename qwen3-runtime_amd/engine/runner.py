@@ -38,6 +38,7 @@ class ModelRunner:
         self.hip_graph = bool(hip_graph) and self.device.type == "cuda"
         self._graphs: dict[tuple, "_DecodeGraph"] = {}
         self._pinned: torch.Tensor | None = None
+        self._copied = torch.cuda.Event() if self.device.type == "cuda" else None
         self.graph_max_batch = 256
 
     # ---- public ------------------------------------------------------------
@@ -74,6 +75,8 @@ class ModelRunner:
         if self.device.type == "cuda":
             if self._pinned is None or self._pinned.numel() < total:
                 self._pinned = torch.empty(max(total, 1 << 16), dtype=torch.int32, pin_memory=True)
+            else:
+                self._copied.synchronize()  # the previous step's copy has left the buffer
             host = self._pinned[:total]
         else:
             host = torch.empty(total, dtype=torch.int32)
@@ -83,8 +86,7 @@ class ModelRunner:
         if self.device.type == "cuda":
             dev = torch.empty(total, dtype=torch.int32, device=self.device)
             dev.copy_(host, non_blocking=True)
-            # the pinned buffer is rewritten by the next step: wait for the copy
-            torch.cuda.current_stream(self.device).synchronize()
+            self._copied.record()
         else:
             dev = host.clone()
         out = {}

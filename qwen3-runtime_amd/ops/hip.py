@@ -69,10 +69,8 @@ class _AttnTileArgs(Structure):
 class _SampleArgs(Structure):
     _fields_ = [
         ("logits", c_void_p), ("work", c_void_p), ("counts", c_void_p), ("slot", c_void_p),
-        ("temperature", c_void_p), ("top_p", c_void_p), ("min_p", c_void_p), ("top_k", c_void_p),
-        ("repetition", c_void_p), ("presence", c_void_p), ("frequency", c_void_p),
-        ("seed", c_void_p), ("draw", c_void_p), ("out_token", c_void_p), ("out_logprob", c_void_p),
-        ("rows", c_int), ("vocab", c_int),
+        ("fparams", c_void_p), ("iparams", c_void_p), ("seeds", c_void_p),
+        ("out_token", c_void_p), ("out_logprob", c_void_p), ("rows", c_int), ("vocab", c_int),
     ]
 
 
@@ -371,32 +369,29 @@ class HipOps:
         self._check(self.lib, self.lib.qrt_argmax(_ptr(logits), _ptr(out), c_int(r), c_int(v), _stream()))
         return out
 
-    def sample(self, logits, params: dict, counts=None):
-        """``params``: device tensors per row: temperature, top_p, min_p, repetition, presence,
-        frequency (float32), top_k, slot (int32), seed, draw (int64). Returns (token, logprob)."""
+    def sample(self, logits, slot, fparams, iparams, seeds, counts=None):
+        """One token per row of ``logits``. Options are read from the row's state slot:
+        ``fparams[slot]`` = temperature, top_p, min_p, repetition, presence, frequency;
+        ``iparams[slot]`` = top_k; ``seeds[slot]`` = seed, index of the next draw (advanced
+        here). Returns (token int32 [R], logprob float32 [R], processed logits [R, V])."""
         _need(logits, "logits", torch.float32)
         r, v = logits.shape
-        f32 = ("temperature", "top_p", "min_p", "repetition", "presence", "frequency")
-        for name in f32:
-            _need(params[name], name, torch.float32, (r,))
-        for name in ("top_k", "slot"):
-            _need(params[name], name, torch.int32, (r,))
-        for name in ("seed", "draw"):
-            _need(params[name], name, torch.int64, (r,))
+        _need(slot, "slot", torch.int32, (r,))
+        n = fparams.shape[0]
+        _need(fparams, "fparams", torch.float32, (n, 8))
+        _need(iparams, "iparams", torch.int32, (n, 2))
+        _need(seeds, "seeds", torch.int64, (n, 2))
         if counts is not None:
-            _need(counts, "counts", torch.int32)
-            if counts.shape[1] != v:
-                raise OpsError(f"counts are {counts.shape[1]} wide for a vocabulary of {v}")
+            _need(counts, "counts", torch.int32, (n, v))
         work = torch.empty_like(logits)
         tok = torch.empty((r,), dtype=torch.int32, device=logits.device)
         lp = torch.empty((r,), dtype=torch.float32, device=logits.device)
         a = _SampleArgs()
-        a.logits, a.work, a.counts = logits.data_ptr(), work.data_ptr(), _addr(counts)
-        for name in f32 + ("top_k", "slot", "seed", "draw"):
-            setattr(a, name, params[name].data_ptr())
+        a.logits, a.work, a.counts, a.slot = logits.data_ptr(), work.data_ptr(), _addr(counts), slot.data_ptr()
+        a.fparams, a.iparams, a.seeds = fparams.data_ptr(), iparams.data_ptr(), seeds.data_ptr()
         a.out_token, a.out_logprob, a.rows, a.vocab = tok.data_ptr(), lp.data_ptr(), r, v
         self._check(self.lib, self.lib.qrt_sample(byref(a), _stream()))
-        return tok, lp
+        return tok, lp, work
 
     def count_tokens(self, counts, slots, tokens):
         _need(counts, "counts", torch.int32)
