@@ -1,0 +1,231 @@
+"""Generation through the entry point on the GPU: greedy tokens equal the plain
+implementation's, batched continuously or alone, from captured graphs or not, with so
+few pages that requests are preempted; the sampler against its plain formulas."""
+
+import math
+
+import pytest
+import torch
+
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def llm(folder, dtype="float32", page=8, pages=64, seqs=4, budget=64, graph=False):
+    from qwen3_runtime_amd.llm import LLM
+
+    return LLM(folder, dtype=dtype, block_size=page, num_kv_blocks=pages, max_num_seqs=seqs,
+               max_num_batched_tokens=budget, cuda_graph=graph)
+
+
+def prompts_for(cfg, lengths, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lengths]
+
+
+@pytest.mark.parametrize("name,lengths,n_out", [("tiny_a", [1, 7, 33, 70], 16), ("tiny_b", [3, 17, 40, 64, 95], 12)])
+def test_greedy_generation_equals_plain(model_folders, tiny_configs, name, lengths, n_out):
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    cfg, w = P.read_model(model_folders[name])
+    prompts = prompts_for(cfg, lengths)
+    want = [P.greedy_generate(cfg, w, p, n_out) for p in prompts]
+    page = tiny_configs[name][1]
+    m = llm(model_folders[name], page=page, pages=80, budget=24)
+    assert m.generate(prompts, SamplingParams(), max_tokens=n_out) == want       # batched together
+    assert [m.generate(p, max_tokens=n_out) for p in prompts] == want            # one after another
+    m.engine.cache.check()
+    assert m.engine.cache.num_free_pages == 80
+
+
+def test_first_tokens_of_a_sequence(model_folders):
+    """Prompts of one and two tokens: position 0 alone, no history at all."""
+    cfg, w = P.read_model(model_folders["tiny_a"])
+    m = llm(model_folders["tiny_a"], page=16)
+    for prompt in ([5], [200, 3]):
+        assert m.generate(prompt, max_tokens=5) == P.greedy_generate(cfg, w, prompt, 5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_equals_eager(model_folders, dtype):
+    cfg, _ = P.read_model(model_folders["tiny_b"])
+    prompts = prompts_for(cfg, [30, 9, 61], seed=3)
+    eager = llm(model_folders["tiny_b"], dtype=dtype, graph=False).generate(prompts, max_tokens=40)
+    m = llm(model_folders["tiny_b"], dtype=dtype, graph=True)
+    assert m.generate(prompts, max_tokens=40) == eager
+    assert m.engine.runner._graphs, "no decode step was replayed from a graph"
+    # replays interleaved with eager work and synchronisation give the same again
+    torch.cuda.synchronize()
+    assert m.generate(prompts, max_tokens=40) == eager
+
+
+def test_preemption_does_not_change_tokens(model_folders):
+    """12 pages of 8 for three requests that need 9 each: some are preempted and recomputed
+    (reference: tests/invariance/test_preempt.py:10-33)."""
+    cfg, w = P.read_model(model_folders["tiny_b"])
+    prompts = prompts_for(cfg, [40, 35, 44], seed=8)
+    want = [P.greedy_generate(cfg, w, p, 24) for p in prompts]
+    m = llm(model_folders["tiny_b"], page=8, pages=12, seqs=3, budget=32)
+    assert m.generate(prompts, max_tokens=24) == want
+    assert m.engine.scheduler.num_preemptions >= 1
+    m.engine.cache.check()
+    assert m.engine.cache.num_free_pages == 12 and m.engine.cache.slots.num_free == 3
+
+
+def test_requests_arriving_mid_decode_and_seeded_sampling(model_folders):
+    """Temperature 0.8 with per-request seeds: tokens do not depend on batch mates or admission time."""
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    cfg, _ = P.read_model(model_folders["tiny_b"])
+    prompts = prompts_for(cfg, [3, 17, 40, 64, 95], seed=1)
+    params = [SamplingParams(temperature=0.8, seed=100 + i) for i in range(5)]
+    m = llm(model_folders["tiny_b"], budget=24, seqs=4, pages=128)
+    alone = [m.engine.generate(p, max_tokens=12, sampling=s) for p, s in zip(prompts, params)]
+    eng = m.engine
+    reqs = [eng.request(eng.add_request(prompts[i], 12, sampling=params[i])) for i in range(2)]
+    for _ in range(5):
+        eng.step()
+    reqs += [eng.request(eng.add_request(prompts[i], 12, sampling=params[i])) for i in range(2, 5)]
+    while not eng.is_finished():
+        eng.step()
+    assert [r.output_tokens for r in reqs] == alone
+    assert all(len(r.logprobs) == 12 and all(lp <= 0 for lp in r.logprobs) for r in reqs)
+    other = m.engine.generate(prompts[2], max_tokens=12, sampling=SamplingParams(temperature=0.8, seed=999))
+    assert other != alone[2]
+
+
+def test_stop_token_and_forced_tokens(model_folders):
+    cfg, w = P.read_model(model_folders["tiny_a"])
+    prompt = prompts_for(cfg, [9], seed=2)[0]
+    want = P.greedy_generate(cfg, w, prompt, 8)
+    eng = llm(model_folders["tiny_a"], page=16).engine
+    out = eng.generate(prompt, max_tokens=8, ignore_eos=False, stop_token_ids=(want[3],))
+    assert out == want[: want.index(want[3]) + 1]
+    forced = [1, 2, 3]
+    rid = eng.add_request(prompt, 5, forced_tokens=forced)
+    req = eng.request(rid)
+    out = list(eng.stream_request(rid))
+    assert out[:3] == forced and len(out) == 5
+    logits = P.forward(cfg, w, prompt)[-1]
+    assert req.logprobs[0] == pytest.approx(float(torch.log_softmax(logits, -1)[1]), abs=1e-4)
+    assert out[3:] == P.greedy_generate(cfg, w, prompt + forced, 2)
+
+
+# ---- the sampling kernel against the plain formulas ---------------------------------------------------
+def sample_rows(logits, rows_params, counts_tokens=None):
+    """Run the device sampler on [R, V] logits with one SamplingParams per row."""
+    from qwen3_runtime_amd.cache import StateSlots
+    from qwen3_runtime_amd.ops.hip import HipOps
+    from qwen3_runtime_amd.sampling.sampler import Sampler
+
+    r, v = logits.shape
+    slots = StateSlots(r, DEV)
+    s = Sampler(HipOps(), slots, v, DEV)
+    for i, (p, seed) in enumerate(rows_params):
+        slot = slots.take(i)
+        s.admit(slot, p, seed, (counts_tokens or {}).get(i, []))
+    slot_rows = torch.tensor([slots.slot(i) for i in range(r)], dtype=torch.int32, device=DEV)
+    return s, slot_rows
+
+
+class _Req:
+    def __init__(self, p):
+        self.sampling = p
+
+    def next_forced_token(self):
+        return None
+
+
+def test_sampler_greedy_ties_and_logprob():
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    x = torch.tensor([[1.0, 3.0, 3.0, 2.0], [0.0, 0.0, 0.0, 0.0], [0.0, 4.0, 1.0, 3.0]], device=DEV)
+    params = [(SamplingParams(), 0), (SamplingParams(temperature=-1.0), 0), (SamplingParams(), 0)]
+    s, rows = sample_rows(x, params)
+    tok, lp = s.sample(x, rows, [_Req(p) for p, _ in params])
+    assert tok == [1, 0, 1]
+    assert lp[2] == pytest.approx(float(torch.log_softmax(x[2].cpu(), -1)[1]), abs=1e-5)
+
+
+def test_sampler_filters_match_plain_and_draws_follow_the_distribution():
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    torch.manual_seed(0)
+    v = 1000
+    base = (torch.randn(v) * 2.0)
+    cases = [
+        SamplingParams(temperature=0.7),
+        SamplingParams(temperature=1.3, top_k=5),
+        SamplingParams(temperature=1.0, top_p=0.6),
+        SamplingParams(temperature=0.9, min_p=0.05),
+        SamplingParams(temperature=1.1, top_k=50, top_p=0.9, min_p=0.01),
+        SamplingParams(temperature=1.0, repetition_penalty=1.7, presence_penalty=0.4, frequency_penalty=0.2),
+    ]
+    seen = [3, 3, 3, 10, 999, 10, 500]
+    n_draws = 4000
+    for p in cases:
+        x = base.clone().double()
+        if p.has_penalties():
+            x = P.apply_penalties(x, seen, p.repetition_penalty, p.presence_penalty, p.frequency_penalty)
+        x = x / p.temperature
+        if p.min_p > 0:
+            x = P.min_p_filter(x, p.min_p)
+        if p.top_k > 0:
+            x = P.top_k_filter(x, p.top_k)
+        if p.top_p < 1:
+            x = P.top_p_filter(x, p.top_p)
+        want = torch.softmax(x, -1)
+        logits = base.to(DEV).repeat(n_draws, 1).contiguous()
+        params = [(p, 1000 + i) for i in range(n_draws)]
+        from qwen3_runtime_amd.cache import StateSlots  # noqa: F401
+
+        s, rows = sample_rows(logits, params, {i: seen for i in range(n_draws)} if p.has_penalties() else None)
+        tok, lp = s.sample(logits, rows, [_Req(p)] * n_draws)
+        tok_t = torch.tensor(tok)
+        assert (want[tok_t] > 0).all(), f"{p}: an id outside the kept set was drawn"
+        freq = torch.bincount(tok_t, minlength=v).double() / n_draws
+        top = torch.topk(want, 5).indices
+        assert (freq[top] - want[top]).abs().max() < 4 * math.sqrt(0.25 / n_draws) + 0.01, str(p)
+        got_lp = torch.tensor(lp).double()
+        torch.testing.assert_close(got_lp, want[tok_t].log(), atol=2e-3, rtol=2e-3)
+
+
+def test_sampler_is_seeded_and_counter_based():
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    torch.manual_seed(1)
+    x = torch.randn(6, 500, device=DEV)
+    p = SamplingParams(temperature=1.0)
+    s1, rows1 = sample_rows(x, [(p, 42)] * 6)
+    a1, _ = s1.sample(x, rows1, [_Req(p)] * 6)
+    a2, _ = s1.sample(x, rows1, [_Req(p)] * 6)        # second draw of the same requests
+    s2, rows2 = sample_rows(x[:3].contiguous(), [(p, 42)] * 3)
+    b1, _ = s2.sample(x[:3].contiguous(), rows2, [_Req(p)] * 3)
+    b2, _ = s2.sample(x[:3].contiguous(), rows2, [_Req(p)] * 3)
+    assert a1[:3] == b1 and a2[:3] == b2               # independent of the batch
+    assert a1 != a2                                    # the draw index advances
+    top1 = SamplingParams(temperature=1.5, top_k=1)
+    s3, rows3 = sample_rows(x, [(top1, 7)] * 6)
+    assert s3.sample(x, rows3, [_Req(top1)] * 6)[0] == torch.argmax(x, -1).tolist()
+
+
+def test_logit_bias_and_penalty_counts_follow_the_output(model_folders):
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    cfg, w = P.read_model(model_folders["tiny_a"])
+    prompt = prompts_for(cfg, [6], seed=4)[0]
+    eng = llm(model_folders["tiny_a"], page=16).engine
+    out = eng.generate(prompt, 3, sampling=SamplingParams(logit_bias={77: 1000.0}))
+    assert out == [77, 77, 77]
+    # a strong frequency penalty forbids repeats: every output differs, and differs from the prompt
+    out = eng.generate(prompt, 20, sampling=SamplingParams(frequency_penalty=1000.0))
+    assert len(set(out)) == 20 and not set(out) & set(prompt)
+    # plain replay of the same rule
+    ids, want = list(prompt), []
+    for _ in range(20):
+        logits = P.apply_penalties(P.forward(cfg, w, ids)[-1], ids, 1.0, 0.0, 1000.0)
+        want.append(P.greedy(logits))
+        ids.append(want[-1])
+    assert out == want

@@ -1,0 +1,335 @@
+"""Each layer part alone against the plain functions, and the generality of the
+assembly: a toy architecture, defined and registered here without touching the
+framework's files, with a mixer that keeps state of its own, another position
+encoding, a windowed attention layer, a layer that runs twice and a step that
+reads another step's cache. It is stepped under every cutting and compared with a
+whole-sequence computation written out below."""
+
+import math
+
+import pytest
+import torch
+
+import traces
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+class DictFetch:
+    """A WeightFetcher over a dict of CPU tensors."""
+
+    def __init__(self, tensors, dtype):
+        from qwen3_runtime_amd.weights.loader import WeightLoader
+
+        class Src:
+            def get(self, name, device="cpu"):
+                # stored in the engine's type, as a model file for that engine would be
+                return tensors[name].to(dtype).to(device)
+
+        self.loader = WeightLoader(Src(), DEV, dtype)
+
+    def __getattr__(self, name):
+        return getattr(self.loader, name)
+
+
+def context(q_lens, kv_lens, dtype, page_size=8, window=None, pages_per_seq=None):
+    """A StepContext and cache pages for sequences processed whole or with history."""
+    from qwen3_runtime_amd.ops.hip import HipOps
+    from qwen3_runtime_amd.parts.base import GroupView, StepContext
+
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    cu, pos, seq = [0], [], []
+    for s, (q, kv) in enumerate(zip(q_lens, kv_lens)):
+        cu.append(cu[-1] + q)
+        pos += list(range(kv - q, kv))
+        seq += [s] * q
+    width = max(-(-kv // page_size) for kv in kv_lens)
+    table = torch.arange(len(q_lens) * width, dtype=torch.int32).view(len(q_lens), width)
+    slots = [int(table[s, p // page_size]) * page_size + p % page_size for s, p in zip(seq, pos)]
+    group = GroupView(page_size, window, table.to(DEV), i32(slots))
+    return StepContext(
+        ops=HipOps(), dtype=dtype, device=torch.device(DEV), num_tokens=len(pos), num_seqs=len(q_lens),
+        positions=i32(pos), cu_q=i32(cu), kv_lens=i32(kv_lens), seq_of_token=i32(seq),
+        state_slots=i32(list(range(len(q_lens)))), first_span=i32([int(q == kv) for q, kv in zip(q_lens, kv_lens)]),
+        q_lens_host=list(q_lens), kv_lens_host=list(kv_lens), max_q_len=max(q_lens), max_kv_len=max(kv_lens),
+        groups=[group]), table.numel()
+
+
+TOL = {torch.float32: dict(atol=2e-5, rtol=2e-5), torch.bfloat16: dict(atol=3e-2, rtol=3e-2)}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_embedding_head_feed_forward_alone(dtype):
+    from qwen3_runtime_amd.parts import build_part
+    from qwen3_runtime_amd.parts.plan import PartSpec
+
+    torch.manual_seed(0)
+    h, inter, v, t = 96, 272, 384, 11
+    w = {"n": 1 + 0.1 * torch.randn(h), "e": 0.5 * torch.randn(v, h), "g": 0.1 * torch.randn(inter, h),
+         "u": 0.1 * torch.randn(inter, h), "d": 0.1 * torch.randn(h, inter)}
+    w = {k: x.to(torch.bfloat16).float() for k, x in w.items()}
+    fetch = DictFetch(w, dtype)
+    ctx, _ = context([t], [t], dtype)
+    ids = torch.randint(0, v, (t,), dtype=torch.int32, device=DEV)
+
+    emb = build_part("embedding", PartSpec("token_embedding", {"vocab_size": v, "hidden_size": h}, {"weight": "e"}))
+    emb.load(fetch)
+    resid = emb.forward(ctx, ids)
+    assert resid.dtype == torch.float32
+    torch.testing.assert_close(resid.cpu(), w["e"][ids.cpu().long()])
+
+    norm = build_part("norm", PartSpec("rmsnorm", {"size": h, "eps": 1e-5}, {"weight": "n"}))
+    norm.load(fetch)
+    delta = (0.3 * torch.randn(t, h)).to(dtype).to(DEV)
+    before = resid.clone()
+    y = norm.forward(ctx, resid, delta)
+    summed = before.cpu().double() + delta.cpu().double()
+    torch.testing.assert_close(resid.cpu().double(), summed, atol=1e-6, rtol=1e-6)   # the add is float32
+    torch.testing.assert_close(y.float().cpu(), P.rms_norm(summed, w["n"].double(), 1e-5).float(), **TOL[dtype])
+
+    ff = build_part("feed_forward", PartSpec("swiglu", {"hidden_size": h, "intermediate_size": inter},
+                                             {"gate": "g", "up": "u", "down": "d"}))
+    ff.load(fetch)
+    x = torch.randn(t, h).to(dtype)
+    want = P.feed_forward(x.double(), {"m.gate_proj.weight": w["g"].double(), "m.up_proj.weight": w["u"].double(),
+                                       "m.down_proj.weight": w["d"].double()}, "m")
+    torch.testing.assert_close(ff.forward(ctx, x.to(DEV)).float().cpu(), want.float(), **TOL[dtype])
+
+    head = build_part("head", PartSpec("linear_head", {"vocab_size": v, "hidden_size": h}, {"weight": "e"}))
+    head.load(fetch)
+    assert head.weight.data_ptr() == emb.weight.data_ptr()      # tied: one tensor
+    logits = head.forward(ctx, x.to(DEV))
+    assert logits.dtype == torch.float32
+    torch.testing.assert_close(logits.cpu(), (x.double() @ w["e"].double().T).float(), **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,d,h,theta,eps", [(4, 2, 16, 64, 1e4, 1e-6), (6, 2, 32, 96, 1e6, 1e-5)])
+def test_attention_mixer_alone(dtype, nq, nkv, d, h, theta, eps):
+    from qwen3_runtime_amd.parts import build_part
+    from qwen3_runtime_amd.parts.base import CacheView
+    from qwen3_runtime_amd.parts.plan import PartSpec
+
+    torch.manual_seed(1)
+    t, ps = 29, 8
+    names = {k: f"a.{k}_proj.weight" for k in "qkvo"} | {"q_norm": "a.q_norm.weight", "k_norm": "a.k_norm.weight"}
+    w = {"a.q_proj.weight": torch.randn(nq * d, h) / 8, "a.k_proj.weight": torch.randn(nkv * d, h) / 8,
+         "a.v_proj.weight": torch.randn(nkv * d, h) / 8, "a.o_proj.weight": torch.randn(h, nq * d) / 8,
+         "a.q_norm.weight": 1 + 0.2 * torch.randn(d), "a.k_norm.weight": 1 + 0.2 * torch.randn(d)}
+    w = {k: x.to(torch.bfloat16).float() for k, x in w.items()}
+    mixer = build_part("mixer", PartSpec("gqa_attention", {
+        "hidden_size": h, "num_heads": nq, "num_kv_heads": nkv, "head_dim": d, "qk_norm_eps": eps,
+        "position": PartSpec("rope_neox", {"head_dim": d, "theta": theta})}, names))
+    for part in (mixer, mixer.position):
+        part.load(DictFetch(w, dtype))
+    ctx, n_pages = context([t], [t], dtype, ps)
+    spec = mixer.cache_spec()
+    cache = CacheView(spec, group=ctx.groups[0],
+                      k=torch.zeros(n_pages, nkv, ps, d, dtype=dtype, device=DEV),
+                      v=torch.zeros(n_pages, nkv, d, ps, dtype=dtype, device=DEV))
+    x = torch.randn(t, h).to(dtype)
+    cfg = dict(num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d, hidden_size=h, rms_norm_eps=eps,
+               rope_theta=theta)
+    want = P.attention_layer(x.double(), {k: v.double() for k, v in w.items()}, "a", cfg, torch.arange(t))
+    got = mixer.forward(ctx, x.to(DEV), cache)
+    torch.testing.assert_close(got.float().cpu(), want.float(), **TOL[dtype])
+
+
+# ------------------------------------------------------------------------------------------------
+# A toy architecture, registered from here.
+# ------------------------------------------------------------------------------------------------
+def register_toy():
+    from qwen3_runtime_amd.parts.base import Mixer, PositionEncoding
+    from qwen3_runtime_amd.parts.plan import CacheSpec, LayerSpec, ModelPlan, PartSpec, RunStep, TensorDecl
+    from qwen3_runtime_amd.registry import register_architecture, register_part
+
+    @register_part("mixer", "toy_ema")
+    class EmaMixer(Mixer):
+        """state <- decay * state + x_t;  y_t = gain * state.  One float32 vector per request."""
+
+        def __init__(self, hidden_size, decay, tensors=None):
+            super().__init__(tensors)
+            self.hidden_size, self.decay, self.gain = hidden_size, decay, None
+
+        def cache_spec(self):
+            return CacheSpec("state", shape=(self.hidden_size,), dtype="float32")
+
+        def tensor_decls(self):
+            return [TensorDecl(self._name("gain"), (self.hidden_size,), init="norm")]
+
+        def load(self, fetch):
+            self.gain = fetch.vector_f32(self._name("gain"))
+
+        def forward(self, ctx, x, cache):
+            out = torch.empty_like(x)
+            slots, row = ctx.state_slots.tolist(), 0
+            for s, n in enumerate(ctx.q_lens_host):          # tokens of a span in order, state carried on
+                state = cache.state[slots[s]]
+                for i in range(row, row + n):
+                    state = self.decay * state + x[i].float()
+                    out[i] = (self.gain * state).to(x.dtype)
+                cache.state[slots[s]] = state
+                row += n
+            return out
+
+    @register_part("position", "toy_scale")
+    class ScalePosition(PositionEncoding):
+        """q and k are scaled by 1 + rate * position: not a rotation, and not fused with anything."""
+
+        def __init__(self, rate, tensors=None):
+            super().__init__(tensors)
+            self.rate = rate
+
+        def rotate(self, ctx, q, k):
+            f = (1.0 + self.rate * ctx.positions.float())[:, None, None]
+            return (q.float() * f).to(q.dtype), (k.float() * f).to(k.dtype)
+
+    def read_config(raw):
+        return dict(raw)
+
+    def make_plan(c):
+        h, d = c["hidden_size"], c["head_dim"]
+
+        def norm(name):
+            return PartSpec("rmsnorm", {"size": h, "eps": c["eps"]}, {"weight": name})
+
+        def attn(i, nq, nkv, position, window=None):
+            p = f"toy.{i}.attn"
+            return PartSpec("gqa_attention", {"hidden_size": h, "num_heads": nq, "num_kv_heads": nkv, "head_dim": d,
+                                              "qk_norm_eps": c["eps"], "position": position, "window": window},
+                            {k: f"{p}.{k}" for k in ("q", "k", "v", "o", "q_norm", "k_norm")})
+
+        def ff(i):
+            return PartSpec("swiglu", {"hidden_size": h, "intermediate_size": c["intermediate_size"]},
+                            {k: f"toy.{i}.ff.{k}" for k in ("gate", "up", "down")})
+
+        def layer(i, mixer):
+            return LayerSpec(PartSpec("pre_norm"), mixer, ff(i),
+                             {"input": norm(f"toy.{i}.norm_in"), "post_mixer": norm(f"toy.{i}.norm_post")})
+
+        rope = PartSpec("rope_neox", {"head_dim": d, "theta": c["theta"]})
+        layers = [
+            layer(0, attn(0, 4, 2, rope)),
+            layer(1, PartSpec("toy_ema", {"hidden_size": h, "decay": 0.7}, {"gain": "toy.1.gain"})),
+            layer(2, attn(2, 2, 1, PartSpec("toy_scale", {"rate": 0.02}), window=c["window"])),
+        ]
+        kv = lambda heads, window=None: CacheSpec("paged_kv", heads=heads, head_dim=d, window=window)
+        caches = [kv(2), CacheSpec("state", shape=(h,), dtype="float32"), kv(1, c["window"]), kv(2)]
+        order = [RunStep(0, 0), RunStep(1, 1), RunStep(2, 2), RunStep(0, 3), RunStep(2, 2, writes_cache=False)]
+        sizes = {"vocab_size": c["vocab_size"], "hidden_size": h}
+        return ModelPlan(h, c["vocab_size"], c["max_positions"],
+                         PartSpec("token_embedding", sizes, {"weight": "toy.embed"}), layers, caches, order,
+                         norm("toy.norm"), PartSpec("linear_head", sizes, {"weight": "toy.head"}))
+
+    register_architecture("ToyMixedForCausalLM", read_config, make_plan)
+
+
+TOY = {"architectures": ["ToyMixedForCausalLM"], "vocab_size": 200, "hidden_size": 48, "head_dim": 16,
+       "intermediate_size": 80, "eps": 1e-5, "theta": 5000.0, "window": 11, "max_positions": 512}
+
+
+def toy_plain(folder, ids):
+    """The toy model on a whole sequence, from the plain functions."""
+    c, w = P.read_model(folder)
+    t = len(ids)
+    pos = torch.arange(t)
+    x = w["toy.embed"][torch.as_tensor(ids)]
+    kept = {}
+
+    def attn(i, nq, nkv, x, scale_pos, window, reuse=False):
+        p, d = f"toy.{i}.attn", c["head_dim"]
+        q = P.rms_norm((x @ w[f"{p}.q"].T).view(t, nq, d), w[f"{p}.q_norm"], c["eps"])
+        if reuse:
+            k, v = kept[i]
+        else:
+            k = P.rms_norm((x @ w[f"{p}.k"].T).view(t, nkv, d), w[f"{p}.k_norm"], c["eps"])
+            v = (x @ w[f"{p}.v"].T).view(t, nkv, d)
+        if scale_pos:
+            f = (1.0 + 0.02 * pos.double())[:, None, None]
+            q = q * f
+            k = k if reuse else k * f
+        else:
+            q = P.rope_neox(q, pos, c["theta"])
+            k = k if reuse else P.rope_neox(k, pos, c["theta"])
+        kept[i] = (k, v)
+        return P.causal_attention(q, k, v, window=window) @ w[f"{p}.o"].T
+
+    def ema(x):
+        state, out = torch.zeros(c["hidden_size"]).double(), []
+        for i in range(t):
+            state = 0.7 * state + x[i]
+            out.append(w["toy.1.gain"] * state)
+        return torch.stack(out)
+
+    def block(i, x, mix):
+        x = x + mix(P.rms_norm(x, w[f"toy.{i}.norm_in"], c["eps"]))
+        n = P.rms_norm(x, w[f"toy.{i}.norm_post"], c["eps"])
+        ffw = {f"f.{k}_proj.weight": w[f"toy.{i}.ff.{k}"] for k in ("gate", "up", "down")}
+        return x + P.feed_forward(n, ffw, "f")
+
+    x = block(0, x, lambda n: attn(0, 4, 2, n, False, None))
+    x = block(1, x, ema)
+    x = block(2, x, lambda n: attn(2, 2, 1, n, True, c["window"]))
+    x = block(0, x, lambda n: attn(0, 4, 2, n, False, None))
+    x = block(2, x, lambda n: attn(2, 2, 1, n, True, c["window"], reuse=True))
+    return P.rms_norm(x, w["toy.norm"], c["eps"]) @ w["toy.head"].T
+
+
+@pytest.fixture(scope="module")
+def toy_folder(tmp_path_factory):
+    from qwen3_runtime_amd.registry import unregister_architecture, unregister_part
+    from qwen3_runtime_amd.weights import write_model_folder
+
+    register_toy()
+    folder = write_model_folder(tmp_path_factory.mktemp("toy"), TOY, seed=21)
+    yield folder
+    unregister_architecture("ToyMixedForCausalLM")
+    unregister_part("mixer", "toy_ema")
+    unregister_part("position", "toy_scale")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail_one_by_one", "portions", "mixed"])
+def test_toy_architecture_under_every_cutting(toy_folder, cut, dtype):
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    reqs = traces.make_requests(TOY["vocab_size"], [5, 37, 64, 90], seed=6)
+    steps = getattr(traces, cut)(reqs)
+    page = 8
+    cfg = EngineConfig(page_size=page, num_pages=traces.peak_tokens(steps) // page, max_num_seqs=4, dtype=dtype,
+                       device=DEV, hip_graph=False)
+    loaded = load(toy_folder, cfg)
+    assert len(loaded.cache.groups) == 2          # two full caches share a pool, the window has its own; state takes no pages
+    got = traces.replay(loaded, steps)
+    want = {}
+    for rid, toks in reqs.items():
+        logits = toy_plain(toy_folder, toks)
+        for p in range(len(toks)):
+            want[(rid, p)] = logits[p].float()
+    tol = dict(atol=5e-5, rtol=5e-5) if dtype == "float32" else dict(atol=4e-2, rtol=4e-2)
+    traces.compare(got, want, **tol)
+
+
+def test_window_layer_gives_pages_back_while_decoding(toy_folder):
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.batch import StepEntry
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg = EngineConfig(page_size=8, num_pages=16, max_num_seqs=2, dtype="float32", device=DEV, hip_graph=False)
+    loaded = load(toy_folder, cfg)
+    cache = loaded.cache
+    win = next(i for i, g in enumerate(cache.groups) if g.window is not None)
+    cache.admit("r")
+    ids = traces.make_requests(TOY["vocab_size"], [100], seed=1)["r0"]
+    got = [loaded.runner.step([StepEntry("r", ids[:60], [59])])[0].cpu()]
+    for p in range(60, 100):
+        got.append(loaded.runner.step([StepEntry("r", ids[p: p + 1], [0])])[0].cpu())
+    held = [p for p in cache.block_table(win, "r") if p >= 0]
+    assert len(held) <= TOY["window"] // 8 + 2 and cache.block_table(win, "r")[0] == -1
+    want = toy_plain(toy_folder, ids)
+    torch.testing.assert_close(torch.stack(got), want[59:].float(), atol=5e-5, rtol=5e-5)
+    cache.release("r")
+    cache.check()
