@@ -194,8 +194,28 @@ class HipOps:
             return torch.matmul(x, w.t())
         out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
         self._check(self.lib, self.lib.qrt_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), F32 if out_f32 else BF16,
-                                                     c_int(m), c_int(n), c_int(k), _stream()))
+                                                     c_int(m), c_int(n), c_int(k), c_int(0), _stream()))
         return out
+
+    # rows up to which the gated activation is fused into the product that follows it
+    fused_act_max_rows = 64
+
+    def swiglu_linear(self, gate_up, w):
+        """``linear(swiglu(gate_up), w)``. With few rows in bfloat16 the activation is computed
+        while the product loads its operand, and the intermediate never reaches memory."""
+        m, two_i = gate_up.shape
+        n, k = w.shape
+        if two_i != 2 * k:
+            raise OpsError(f"swiglu_linear: gate_up is {tuple(gate_up.shape)}, weight is {tuple(w.shape)}")
+        if (gate_up.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and m <= self.fused_act_max_rows
+                and k % 32 == 0):
+            _need(gate_up, "gate_up")
+            _need(w, "weight")
+            out = torch.empty((m, n), dtype=torch.bfloat16, device=gate_up.device)
+            self._check(self.lib, self.lib.qrt_gemm_bf16(_ptr(gate_up), _ptr(w), _ptr(out), BF16, c_int(m),
+                                                         c_int(n), c_int(k), c_int(1), _stream()))
+            return out
+        return self.linear(self.swiglu(gate_up), w)
 
     # ---- q/k norm, rotation, cache write ----------------------------------------
     def _qk(self, args: _QkArgs, dtype, num_pages=0):

@@ -36,5 +36,4 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx, x):
         gate_up = ctx.ops.linear(x, self.gate_up)
-        act = ctx.ops.swiglu(gate_up)
-        return ctx.ops.linear(act, self.down)
+        return ctx.ops.swiglu_linear(gate_up, self.down)

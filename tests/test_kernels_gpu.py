@@ -98,6 +98,27 @@ def test_gemm_bf16(ops, m, n, k, out_f32):
         close(got, want, 2e-2, 2e-2)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 2560, 9728), (8, 96, 288), (33, 100, 64), (64, 272, 96), (70, 64, 64),
+                                   (5, 64, 48)])
+def test_swiglu_linear(ops, m, n, k):
+    """The fused form (few rows) and the two-kernel form agree with the plain one."""
+    for dtype in (torch.bfloat16, torch.float32):
+        gu, w = rnd(m, 2 * k, dtype=dtype, seed=3, scale=2.0), rnd(n, k, dtype=dtype, seed=4, scale=0.05)
+        act = R.swiglu(gu.double())
+        want = act @ w.double().T
+        tol = 3e-2 if dtype == torch.bfloat16 else 1e-4
+        close(ops.swiglu_linear(gu, w), want, tol * max(1.0, float(want.abs().max())), tol)
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 40, 64])
+@pytest.mark.parametrize("n,k", [(6144, 2560), (2560, 4096), (1000, 9728), (272, 96)])
+def test_gemm_bf16_few_rows_at_model_sizes(ops, m, n, k):
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.02)
+    want = x.double() @ w.double().T
+    close(ops.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
+    close(ops.linear(x, w), want, 3e-2, 3e-2)
+
+
 def test_gemm_bf16_large_uses_blas_and_agrees(ops):
     x, w = rnd(300, 512, dtype=torch.bfloat16, seed=1), rnd(640, 512, dtype=torch.bfloat16, seed=2, scale=0.05)
     close(ops.linear(x, w), x.double() @ w.double().T, 3e-2, 3e-2)
