@@ -90,130 +90,141 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 
 // ---------------------------------------------------------------- few rows
 // M <= 64 (decoding): the product is a stream of the weight matrix, so the
-// layout is chosen for memory parallelism, not for reuse. A block owns 16
-// weight rows (one MFMA tile of outputs n) and all of K; its NW waves take the
-// 32-wide k-steps round-robin, so that in every round the block reads
-// 16 rows x NW x 64 contiguous bytes. Each wave keeps MB accumulators (16 rows
-// of M each); activations come from L2/L1 (they are tiny), optionally as
-// silu(gate) * up of a [M, 2K] input. Partial sums meet in LDS and are added in
-// wave order, so the result does not depend on timing.
-template <bool SWIGLU>
-__device__ __forceinline__ bf16x8_t load_act(const bf16_t* __restrict__ row, int k, int K, bool valid) {
-  bf16x8_t v;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) v[e] = (bf16_t)0.0f;
-  if (!valid) return v;
-  if (!SWIGLU) return *(const bf16x8_t*)(row + k);
-  const bf16x8_t g = *(const bf16x8_t*)(row + k);
-  const bf16x8_t u = *(const bf16x8_t*)(row + K + k);
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float gf = (float)g[e];
-    v[e] = (bf16_t)(gf / (1.0f + __expf(-gf)) * (float)u[e]);
-  }
-  return v;
-}
-
-template <int MB, int NW, bool SWIGLU, typename TO>
+// layout is chosen for memory parallelism, not for reuse. A block owns NT
+// tiles of 16 weight rows and all of K; its NW waves take the 32-wide k-steps
+// round-robin, so that in every round the block reads 16 rows x NW x 64
+// contiguous bytes per tile. A wave issues the loads of U steps before the
+// first MFMA of them. Each wave keeps MB accumulators (16 rows of M each) per
+// tile; activations come from L2/L1 (they are tiny). Partial sums meet in LDS
+// and are added in wave order, so the result does not depend on timing.
+//
+// GATED: W holds 2N rows, gate rows then up rows; the block owns matching
+// tiles of both and writes silu(gate) * up, so the gated feed-forward's
+// intermediate [M, 2N] never reaches memory.
+template <int MB, int NW, int NT, int U, bool GATED, typename TO>
 __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A,
                                                                     const bf16_t* __restrict__ W,
                                                                     TO* __restrict__ C, int M, int N, int K) {
-  extern __shared__ float red[];  // [NW][MB][4][64]
+  constexpr int WT = GATED ? 2 * NT : NT;  // weight tiles per block
+  extern __shared__ float red[];            // [NW][WT][MB][4][64]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int n = n0 + r16;
-  const bf16_t* wrow = W + (size_t)(n < N ? n : N - 1) * K;
-  const int a_stride = SWIGLU ? 2 * K : K;
+  const int n0 = blockIdx.x * 16 * NT;
+  const bf16_t* wrow[WT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int n = min(n0 + 16 * t + r16, N - 1);
+    wrow[t] = W + (size_t)n * K + 8 * quad;
+    if (GATED) wrow[NT + t] = W + (size_t)(N + n) * K + 8 * quad;
+  }
   const bf16_t* arow[MB];
   bool avalid[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
     const int m = 16 * b + r16;
     avalid[b] = m < M;
-    arow[b] = A + (size_t)(avalid[b] ? m : 0) * a_stride;
+    arow[b] = A + (size_t)(avalid[b] ? m : 0) * K + 8 * quad;
   }
-  f32x4_t acc[MB];
+  f32x4_t acc[WT][MB];
 #pragma unroll
-  for (int b = 0; b < MB; ++b) acc[b] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < WT; ++t)
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[t][b] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
   const int steps = K >> 5;  // K is a multiple of 32 here
-  constexpr int U = 4;
-  int s = wave;
-  for (; s + (U - 1) * NW < steps; s += U * NW) {
-    bf16x8_t w[U];
+  bf16x8_t zero;
 #pragma unroll
-    for (int u = 0; u < U; ++u) w[u] = *(const bf16x8_t*)(wrow + ((s + u * NW) << 5) + 8 * quad);
+  for (int e = 0; e < 8; ++e) zero[e] = (bf16_t)0.0f;
+  for (int s0 = wave; s0 < steps; s0 += U * NW) {
+    bf16x8_t w[U][WT], a[U][MB];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = ((s + u * NW) << 5) + 8 * quad;
+      const int s = s0 + u * NW;
+      if (s < steps) {  // uniform over the wave
 #pragma unroll
-      for (int b = 0; b < MB; ++b) {
-        const bf16x8_t a = load_act<SWIGLU>(arow[b], k, K, avalid[b]);
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], a, acc[b], 0, 0, 0);
+        for (int t = 0; t < WT; ++t) w[u][t] = *(const bf16x8_t*)(wrow[t] + (s << 5));
+#pragma unroll
+        for (int b = 0; b < MB; ++b) a[u][b] = avalid[b] ? *(const bf16x8_t*)(arow[b] + (s << 5)) : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (s0 + u * NW < steps) {
+#pragma unroll
+        for (int t = 0; t < WT; ++t)
+#pragma unroll
+          for (int b = 0; b < MB; ++b)
+            acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][t], a[u][b], acc[t][b], 0, 0, 0);
       }
     }
   }
-  for (; s < steps; s += NW) {
-    const int k = (s << 5) + 8 * quad;
-    const bf16x8_t w = *(const bf16x8_t*)(wrow + k);
-#pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      const bf16x8_t a = load_act<SWIGLU>(arow[b], k, K, avalid[b]);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, a, acc[b], 0, 0, 0);
-    }
-  }
 
 #pragma unroll
-  for (int b = 0; b < MB; ++b)
+  for (int t = 0; t < WT; ++t)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[((wave * MB + b) * 4 + r) * 64 + lane] = acc[b][r];
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[(((wave * WT + t) * MB + b) * 4 + r) * 64 + lane] = acc[t][b][r];
   __syncthreads();
-  // thread t < MB * 64 finishes accumulator block b = t / 64 of lane t % 64
-  for (int t = threadIdx.x; t < MB * 64; t += 64 * NW) {
-    const int b = t >> 6, l = t & 63;
+  // one thread per (tile, accumulator block, lane) adds the waves' parts in order
+  for (int i = threadIdx.x; i < NT * MB * 64; i += 64 * NW) {
+    const int l = i & 63, b = (i >> 6) % MB, t = (i >> 6) / MB;
     const int m = 16 * b + (l & 15);
-    const int nn = n0 + 4 * (l >> 4);
-    float sum[4];
+    const int nn = n0 + 16 * t + 4 * (l >> 4);
+    float sum[4], sum2[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float v = 0.f;
-      for (int w = 0; w < NW; ++w) v += red[((w * MB + b) * 4 + r) * 64 + l];
+      float v = 0.f, v2 = 0.f;
+      for (int w = 0; w < NW; ++w) {
+        v += red[(((w * WT + t) * MB + b) * 4 + r) * 64 + l];
+        if (GATED) v2 += red[(((w * WT + NT + t) * MB + b) * 4 + r) * 64 + l];
+      }
       sum[r] = v;
+      sum2[r] = v2;
     }
     if (m < M) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (nn + r < N) C[(size_t)m * N + nn + r] = from_f32<TO>(sum[r]);
+      for (int r = 0; r < 4; ++r) {
+        if (nn + r < N) {
+          // the gate and the up value are rounded to bfloat16 first, as the unfused kernels see them
+          const float g = (float)(bf16_t)sum[r];
+          const float out = GATED ? g / (1.0f + expf(-g)) * (float)(bf16_t)sum2[r] : sum[r];
+          C[(size_t)m * N + nn + r] = from_f32<TO>(out);
+        }
+      }
     }
   }
 }
 
-template <int MB, int NW, bool SWIGLU>
+template <int MB, int NW, int NT, int U, bool GATED>
 static int launch_skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K,
                          hipStream_t stream) {
-  dim3 grid((N + 15) / 16), block(64 * NW);
-  const size_t smem = (size_t)NW * MB * 4 * 64 * sizeof(float);
+  dim3 grid((N + 16 * NT - 1) / (16 * NT)), block(64 * NW);
+  const size_t smem = (size_t)NW * (GATED ? 2 : 1) * NT * MB * 4 * 64 * sizeof(float);
   if (out_dtype == QRT_BF16)
-    gemm_bf16_skinny_kernel<MB, NW, SWIGLU, bf16_t><<<grid, block, smem, stream>>>(a, w, (bf16_t*)c, M, N, K);
+    gemm_bf16_skinny_kernel<MB, NW, NT, U, GATED, bf16_t><<<grid, block, smem, stream>>>(a, w, (bf16_t*)c, M, N, K);
   else if (out_dtype == QRT_F32)
-    gemm_bf16_skinny_kernel<MB, NW, SWIGLU, float><<<grid, block, smem, stream>>>(a, w, (float*)c, M, N, K);
+    gemm_bf16_skinny_kernel<MB, NW, NT, U, GATED, float><<<grid, block, smem, stream>>>(a, w, (float*)c, M, N, K);
   else
     return qrt_fail("gemm_bf16: unknown output dtype %d", out_dtype);
   QRT_LAUNCH_CHECK("gemm_bf16_skinny");
   return 0;
 }
 
-template <bool SWIGLU>
+template <bool GATED>
 static int skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K, hipStream_t st) {
-  // more waves per block when there are few blocks or K is long
-  const bool many = (N / 16 < 512) || (K >= 8192);
-  if (M <= 16) return many ? launch_skinny<1, 16, SWIGLU>(a, w, c, out_dtype, M, N, K, st)
-                           : launch_skinny<1, 8, SWIGLU>(a, w, c, out_dtype, M, N, K, st);
-  if (M <= 32) return many ? launch_skinny<2, 16, SWIGLU>(a, w, c, out_dtype, M, N, K, st)
-                           : launch_skinny<2, 8, SWIGLU>(a, w, c, out_dtype, M, N, K, st);
-  return many ? launch_skinny<4, 16, SWIGLU>(a, w, c, out_dtype, M, N, K, st)
-              : launch_skinny<4, 8, SWIGLU>(a, w, c, out_dtype, M, N, K, st);
+  const int tiles = (N + 15) / 16;
+  if (M <= 16) {
+    if (tiles >= 2048) return launch_skinny<1, 8, 2, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
+    if (tiles >= 512 || K < 4096) return launch_skinny<1, 8, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
+    return launch_skinny<1, 16, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
+  }
+  if (M <= 32) {
+    if (tiles >= 512) return launch_skinny<2, 8, 2, 4, GATED>(a, w, c, out_dtype, M, N, K, st);
+    return launch_skinny<2, 8, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
+  }
+  if (tiles >= 512 && !GATED) return launch_skinny<4, 8, 2, 2, GATED>(a, w, c, out_dtype, M, N, K, st);
+  return launch_skinny<4, 8, 1, 4, GATED>(a, w, c, out_dtype, M, N, K, st);
 }
 
 template <int MT, int NT>
@@ -230,18 +241,19 @@ static int launch(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int 
   return 0;
 }
 
-// act: 0 = A is [M, K]; 1 = A is [M, 2K] and the operand is silu(A[:, :K]) * A[:, K:]
-extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K, int act,
+// gated = 0: C[M, N] = A W^T with W [N, K].
+// gated = 1: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A Wg^T) * (A Wu^T).
+extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K, int gated,
                              hipStream_t stream) {
   QRT_CHECK(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
-  QRT_CHECK(act == 0 || act == 1, "gemm_bf16: unknown activation %d", act);
+  QRT_CHECK(gated == 0 || gated == 1, "gemm_bf16: unknown mode %d", gated);
   if (M == 0) return 0;
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
   const bool aligned = (K % 32 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
-  if (M <= 64 && aligned) return act ? skinny<true>(A, W, c, out_dtype, M, N, K, stream)
-                                     : skinny<false>(A, W, c, out_dtype, M, N, K, stream);
-  QRT_CHECK(act == 0, "gemm_bf16: the fused activation needs M <= 64 and K a multiple of 32 (M=%d K=%d)", M, K);
+  if (M <= 64 && aligned) return gated ? skinny<true>(A, W, c, out_dtype, M, N, K, stream)
+                                       : skinny<false>(A, W, c, out_dtype, M, N, K, stream);
+  QRT_CHECK(gated == 0, "gemm_bf16: the gated form needs M <= 64 and K a multiple of 32 (M=%d K=%d)", M, K);
   if (M <= 16) return launch<1, 2>(A, W, c, out_dtype, M, N, K, stream);
   if (M <= 32) return launch<2, 2>(A, W, c, out_dtype, M, N, K, stream);
   return launch<4, 4>(A, W, c, out_dtype, M, N, K, stream);

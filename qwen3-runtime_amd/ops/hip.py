@@ -197,25 +197,26 @@ class HipOps:
                                                      c_int(m), c_int(n), c_int(k), c_int(0), _stream()))
         return out
 
-    # rows up to which the gated activation is fused into the product that follows it
-    fused_act_max_rows = 64
+    # rows up to which the gated activation is fused into the product before it
+    fused_gate_max_rows = 64
 
-    def swiglu_linear(self, gate_up, w):
-        """``linear(swiglu(gate_up), w)``. With few rows in bfloat16 the activation is computed
-        while the product loads its operand, and the intermediate never reaches memory."""
-        m, two_i = gate_up.shape
-        n, k = w.shape
-        if two_i != 2 * k:
-            raise OpsError(f"swiglu_linear: gate_up is {tuple(gate_up.shape)}, weight is {tuple(w.shape)}")
-        if (gate_up.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and m <= self.fused_act_max_rows
+    def gated_linear(self, x, w_gate_up):
+        """``swiglu(linear(x, w_gate_up))`` with ``w_gate_up`` [2I, K], gate rows first. With few
+        rows in bfloat16 one kernel forms both halves and applies the activation in its epilogue,
+        so the [T, 2I] intermediate never reaches memory."""
+        m, k = x.shape
+        two_i, kw = w_gate_up.shape
+        if k != kw or two_i % 2:
+            raise OpsError(f"gated_linear: x is {tuple(x.shape)}, weight is {tuple(w_gate_up.shape)}")
+        if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and m <= self.fused_gate_max_rows
                 and k % 32 == 0):
-            _need(gate_up, "gate_up")
-            _need(w, "weight")
-            out = torch.empty((m, n), dtype=torch.bfloat16, device=gate_up.device)
-            self._check(self.lib, self.lib.qrt_gemm_bf16(_ptr(gate_up), _ptr(w), _ptr(out), BF16, c_int(m),
-                                                         c_int(n), c_int(k), c_int(1), _stream()))
+            _need(x, "x")
+            _need(w_gate_up, "weight")
+            out = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
+            self._check(self.lib, self.lib.qrt_gemm_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), BF16, c_int(m),
+                                                         c_int(two_i // 2), c_int(k), c_int(1), _stream()))
             return out
-        return self.linear(self.swiglu(gate_up), w)
+        return self.swiglu(self.linear(x, w_gate_up))
 
     # ---- q/k norm, rotation, cache write ----------------------------------------
     def _qk(self, args: _QkArgs, dtype, num_pages=0):

@@ -35,5 +35,5 @@ class SwiGLU(FeedForward):
         self.down = fetch.matrix(self._name("down"))
 
     def forward(self, ctx, x):
-        gate_up = ctx.ops.linear(x, self.gate_up)
-        return ctx.ops.swiglu_linear(gate_up, self.down)
+        act = ctx.ops.gated_linear(x, self.gate_up)
+        return ctx.ops.linear(act, self.down)

@@ -184,8 +184,8 @@ class TorchOps:
     def swiglu(self, gate_up):
         return swiglu(gate_up, self.compute)
 
-    def swiglu_linear(self, gate_up, w):
-        return linear(swiglu(gate_up, self.compute), w, False, self.compute)
+    def gated_linear(self, x, w_gate_up):
+        return swiglu(linear(x, w_gate_up, False, self.compute), self.compute)
 
     def argmax(self, logits):
         return argmax(logits)

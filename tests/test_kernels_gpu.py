@@ -98,16 +98,20 @@ def test_gemm_bf16(ops, m, n, k, out_f32):
         close(got, want, 2e-2, 2e-2)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 2560, 9728), (8, 96, 288), (33, 100, 64), (64, 272, 96), (70, 64, 64),
-                                   (5, 64, 48)])
-def test_swiglu_linear(ops, m, n, k):
+@pytest.mark.parametrize("m,i,k", [(1, 9728, 2560), (8, 288, 96), (33, 100, 64), (64, 272, 96), (70, 64, 64),
+                                   (5, 64, 48), (16, 1000, 128)])
+def test_gated_linear(ops, m, i, k):
     """The fused form (few rows) and the two-kernel form agree with the plain one."""
     for dtype in (torch.bfloat16, torch.float32):
-        gu, w = rnd(m, 2 * k, dtype=dtype, seed=3, scale=2.0), rnd(n, k, dtype=dtype, seed=4, scale=0.05)
-        act = R.swiglu(gu.double())
-        want = act @ w.double().T
+        x, w = rnd(m, k, dtype=dtype, seed=3), rnd(2 * i, k, dtype=dtype, seed=4, scale=0.05)
+        gu = x.double() @ w.double().T
+        if dtype == torch.bfloat16:
+            gu = gu.to(torch.bfloat16).double()     # the unfused kernels round here
+        want = R.swiglu(gu)
         tol = 3e-2 if dtype == torch.bfloat16 else 1e-4
-        close(ops.swiglu_linear(gu, w), want, tol * max(1.0, float(want.abs().max())), tol)
+        got = ops.gated_linear(x, w)
+        assert got.shape == (m, i)
+        close(got, want, tol, tol)
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 40, 64])
