@@ -10,7 +10,8 @@
 //
 // Products. Scores are formed transposed, S^T = K Q^T, with the 16x16x32 MFMA:
 // the A operand is 16 keys x 32 head elements read straight from the key page,
-// the B operand 32 head elements x 16 rows of Q held in registers. The 16 key
+// the B operand 32 head elements x 16 rows of Q held in registers (a head size
+// with a 16-wide remainder pads that step with zeros). The 16 key
 // rows of the two MFMAs that cover a block of 32 keys are permuted (row
 // 4 quad + r of sub-block kb holds key 8 quad + 4 kb + r) so that each lane ends
 // up with the scores of 8 consecutive keys for its row: exactly the B operand
@@ -33,7 +34,18 @@
 #error "QRT_HEAD_DIM must be a multiple of 16 between 16 and 512"
 #endif
 
-typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+// 8 head elements from ``p`` for the quads that hold real data, zeros for the others: a head
+// size with a 16-wide remainder runs the 32-wide MFMA with the upper half of the step empty.
+// (A 16x16x16 MFMA chained onto the 16x16x32 ones for that remainder gave results that
+// differed from run to run; one MFMA shape per accumulator chain does not.)
+__device__ __forceinline__ bf16x8_t load_tail(const bf16_t* p, int quad) {
+  bf16x8_t v;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (bf16_t)0.0f;
+  if (quad < 2) v = *(const bf16x8_t*)(p + 8 * quad);
+  return v;
+}
 
 struct AttnTileArgs {
   const bf16_t* q;        // [T, nq * D]
@@ -83,8 +95,8 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnTileArgs a) {
   bf16x8_t qreg[KFULL > 0 ? KFULL : 1];
 #pragma unroll
   for (int i = 0; i < KFULL; ++i) qreg[i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
-  s16x4_t qtail = {0, 0, 0, 0};
-  if (KTAIL) qtail = *(const s16x4_t*)(qp + 32 * KFULL + 4 * quad);
+  bf16x8_t qtail = load_tail(qp, 2);  // zeros
+  if (KTAIL) qtail = load_tail(qp + 32 * KFULL, quad);
 
   // keys this wave may need: [lo, pos_max]
   const int row_last = min(row0 + 15, n_rows - 1);
@@ -116,8 +128,8 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnTileArgs a) {
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk, qreg[i], acc, 0, 0, 0);
       }
       if (KTAIL) {
-        const s16x4_t kk = *(const s16x4_t*)(kp + 32 * KFULL + 4 * quad);
-        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kk, qtail, acc, 0, 0, 0);
+        const bf16x8_t kk = load_tail(kp + 32 * KFULL, quad);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk, qtail, acc, 0, 0, 0);
       }
       s[kb] = acc;
     }
@@ -209,6 +221,283 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
     }
     out[row * D + d] = (bf16_t)(wsum > 0.f ? acc / wsum : 0.f);
   }
+}
+
+// ------------------------------------------------------------------ decoding
+// Tiles of at most 16 rows (a decoded token's g query heads, or a very short
+// portion): one block of DW waves per (tile, key head, split). The waves take the
+// block's 32-key blocks round-robin, each with its own running maximum, sum and
+// accumulator; the next block's keys and values are loaded while the current one
+// is multiplied, and page numbers are fetched one block further ahead, so that no
+// load waits for another. The waves' results meet in LDS. With several splits each
+// block writes its normalised part and the base-2 log of its sum; the block that
+// arrives last at the tile's counter merges the parts and resets the counter, so
+// no second launch and no clearing between launches is needed.
+constexpr int DW = 4;
+
+struct KvBlock {  // the keys of one block, as MFMA operands
+  bf16x8_t k[2][KFULL > 0 ? KFULL : 1];
+  bf16x8_t kt[2];
+};
+
+struct DecodeArgs {
+  AttnTileArgs t;
+  int* counters;  // [num_tiles * nkv], zero before the first launch; left zero by every launch
+};
+
+__device__ __forceinline__ void block_pages(const int* __restrict__ table, int base, int lo, int pos_max, int ps,
+                                            int r16, int quad, int pg[3]) {
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
+    pg[kb] = table[kidx / ps];
+  }
+  const int kv0 = base + 8 * quad;
+  pg[2] = (kv0 <= pos_max && kv0 + 7 >= lo) ? table[kv0 / ps] : -1;
+}
+
+__device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int base, int lo, int pos_max, int r16,
+                                           int quad, const int pg[3], KvBlock& blk) {
+  const int ps = a.page_size;
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
+    const bf16_t* kp = a.k_cache + (((size_t)pg[kb] * a.nkv + kvh) * ps + (kidx % ps)) * D;
+#pragma unroll
+    for (int i = 0; i < KFULL; ++i) blk.k[kb][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
+    if (KTAIL) blk.kt[kb] = load_tail(kp + 32 * KFULL, quad);
+  }
+}
+
+__device__ __forceinline__ void block_load_values(const AttnTileArgs& a, int kvh, int base, int r16, int quad,
+                                                  int vpage, bf16x8_t* v) {
+  const int ps = a.page_size;
+  const int kv0 = base + 8 * quad;
+  const bool vload = vpage >= 0;
+  const bf16_t* vp = a.v_cache + (((size_t)(vload ? vpage : 0) * a.nkv + kvh) * D + r16) * ps + (kv0 % ps);
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    if (vload) v[i] = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
+    else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] = (bf16_t)0.0f;
+    }
+  }
+}
+
+__device__ __forceinline__ void block_compute(const KvBlock& blk, const bf16x8_t* v, const bf16x8_t* qreg,
+                                              bf16x8_t qtail, int base, int quad, bool row_valid, int qpos,
+                                              int window, float scale_log2, float& m, float& l, f32x4_t* o) {
+  f32x4_t s[2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < KFULL; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[kb][i], qreg[i], acc, 0, 0, 0);
+    if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kt[kb], qtail, acc, 0, 0, 0);
+    s[kb] = acc;
+  }
+  float p[8];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int key = base + 8 * quad + e;
+    const bool vis = row_valid && key <= qpos && (window == 0 || key > qpos - window);
+    p[e] = vis ? s[e >> 2][e & 3] * scale_log2 : -INFINITY;
+    mx = fmaxf(mx, p[e]);
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(m, mx);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;
+  const float corr = exp2f(m - m_use);
+  float psum = 0.f;
+  bf16x8_t pb;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float pe = exp2f(p[e] - m_use);
+    psum += pe;
+    pb[e] = (bf16_t)pe;
+  }
+  l = l * corr + psum;
+  m = m_new;
+#pragma unroll
+  for (int i = 0; i < DB; ++i) {
+    o[i] *= corr;
+    o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v[i], pb, o[i], 0, 0, 0);
+  }
+}
+
+__global__ __launch_bounds__(64 * DW) void attention_bf16_decode_kernel(DecodeArgs da) {
+  const AttnTileArgs& a = da.t;
+  // per wave: maximum and sum per row, unnormalised accumulator [16][D]
+  extern __shared__ float lds[];
+  float* lds_m = lds;                 // [DW][16]
+  float* lds_l = lds + DW * 16;       // [DW][16]
+  float* lds_o = lds + 2 * DW * 16;   // [DW][16][D]
+  __shared__ int is_last;
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int seq = a.tile_seq[blockIdx.x];
+  const int kvh = blockIdx.y, split = blockIdx.z;
+  const int g = a.nq / a.nkv;
+  const int q_begin = a.cu_q[seq];
+  const int q_len = a.cu_q[seq + 1] - q_begin;
+  const int kv_len = a.kv_lens[seq];
+  const int n_rows = q_len * g;  // <= 16 by the launch condition
+  const int first_pos = kv_len - q_len;
+  const bool row_valid = r16 < n_rows;
+  const int row_c = row_valid ? r16 : max(n_rows - 1, 0);
+  const int tok = row_c / g, hg = row_c - tok * g;
+  const int qpos = first_pos + tok;
+  const int head = kvh * g + hg;
+  const int* table = a.block_table + (size_t)seq * a.table_width;
+
+  f32x4_t o[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) o[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  if (n_rows > 0) {
+    const bf16_t* qp = a.q + ((size_t)(q_begin + tok) * a.nq + head) * D;
+    bf16x8_t qreg[KFULL > 0 ? KFULL : 1];
+#pragma unroll
+    for (int i = 0; i < KFULL; ++i) qreg[i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
+    bf16x8_t qtail = load_tail(qp, 2);  // zeros
+    if (KTAIL) qtail = load_tail(qp + 32 * KFULL, quad);
+
+    const int pos_min = first_pos, pos_max = first_pos + (n_rows - 1) / g;
+    const int lo = a.window > 0 ? max(0, pos_min - a.window + 1) : 0;
+    const int blk_begin = lo >> 5, blk_end = (pos_max >> 5) + 1;
+    const int per = (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
+    const int b0 = blk_begin + split * per;
+    const int b1 = min(blk_end, b0 + per);
+
+    // keys are loaded one block ahead, page numbers two; values at the top of their block
+    KvBlock A, B;
+    bf16x8_t v[DB];
+    int pgA[3], pgB[3];
+    int b = b0 + wave;
+    if (b < b1) {
+      block_pages(table, b << 5, lo, pos_max, a.page_size, r16, quad, pgA);
+      block_load(a, kvh, b << 5, lo, pos_max, r16, quad, pgA, A);
+    }
+    if (b + DW < b1) block_pages(table, (b + DW) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
+    while (b < b1) {
+      const int vpa = pgA[2];
+      if (b + DW < b1) block_load(a, kvh, (b + DW) << 5, lo, pos_max, r16, quad, pgB, B);
+      block_load_values(a, kvh, b << 5, r16, quad, vpa, v);
+      if (b + 2 * DW < b1) block_pages(table, (b + 2 * DW) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
+      block_compute(A, v, qreg, qtail, b << 5, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+      b += DW;
+      if (b >= b1) break;
+      const int vpb = pgB[2];
+      if (b + DW < b1) block_load(a, kvh, (b + DW) << 5, lo, pos_max, r16, quad, pgA, A);
+      block_load_values(a, kvh, b << 5, r16, quad, vpb, v);
+      if (b + 2 * DW < b1) block_pages(table, (b + 2 * DW) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
+      block_compute(B, v, qreg, qtail, b << 5, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+      b += DW;
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+
+  // the waves' parts meet in LDS
+  if (quad == 0) {
+    lds_m[wave * 16 + r16] = m;
+    lds_l[wave * 16 + r16] = l;
+  }
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) lds_o[(wave * 16 + r16) * D + 16 * i + 4 * quad + r] = o[i][r];
+  __syncthreads();
+
+  const size_t tile_row0 = (size_t)q_begin * a.nq;  // rows of this sequence start here, in units of heads
+  for (int idx = threadIdx.x; idx < 16 * D; idx += 64 * DW) {
+    const int row = idx / D, d = idx - row * D;
+    if (row >= n_rows) continue;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DW; ++w) mm = fmaxf(mm, lds_m[w * 16 + row]);
+    float num = 0.f, den = 0.f;
+    if (mm != -INFINITY) {
+#pragma unroll
+      for (int w = 0; w < DW; ++w) {
+        const float f = exp2f(lds_m[w * 16 + row] - mm);
+        num += f * lds_o[(w * 16 + row) * D + d];
+        den += f * lds_l[w * 16 + row];
+      }
+    }
+    const int rt = row / g, rh = row - rt * g;
+    const size_t row_index = tile_row0 + (size_t)rt * a.nq + kvh * g + rh;
+    const float val = den > 0.f ? num / den : 0.f;
+    if (a.num_splits == 1) {
+      a.out[row_index * D + d] = (bf16_t)val;
+    } else {
+      a.part_o[(row_index * a.num_splits + split) * D + d] = val;
+      if (d == 0) a.part_lse[row_index * a.num_splits + split] = den > 0.f ? mm + log2f(den) : -INFINITY;
+    }
+  }
+  if (a.num_splits == 1) return;
+
+  // the last block of this (tile, key head) to get here merges all parts
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int* c = da.counters + (size_t)blockIdx.x * a.nkv + kvh;
+    const int prev = atomicAdd(c, 1);
+    is_last = prev == a.num_splits - 1;
+    if (is_last) *c = 0;  // nobody else touches it any more in this launch
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+  for (int idx = threadIdx.x; idx < 16 * D; idx += 64 * DW) {
+    const int row = idx / D, d = idx - row * D;
+    if (row >= n_rows) continue;
+    const int rt = row / g, rh = row - rt * g;
+    const size_t row_index = tile_row0 + (size_t)rt * a.nq + kvh * g + rh;
+    const float* lse = a.part_lse + row_index * a.num_splits;
+    float mm = -INFINITY;
+    for (int sidx = 0; sidx < a.num_splits; ++sidx)
+      mm = fmaxf(mm, __hip_atomic_load(lse + sidx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    float num = 0.f, den = 0.f;
+    if (mm != -INFINITY) {
+      for (int sidx = 0; sidx < a.num_splits; ++sidx) {
+        const float f = exp2f(__hip_atomic_load(lse + sidx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - mm);
+        den += f;
+        num += f * __hip_atomic_load(a.part_o + (row_index * a.num_splits + sidx) * D + d, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    a.out[row_index * D + d] = (bf16_t)(den > 0.f ? num / den : 0.f);
+  }
+}
+
+// tiles must all have at most 16 rows (max_q_len * g <= 16) and D <= 256
+extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int* counters, int num_counters,
+                                         hipStream_t stream) {
+  DecodeArgs da;
+  da.t = *args;
+  da.counters = counters;
+  const AttnTileArgs& a = da.t;
+  QRT_CHECK(a.nq > 0 && a.nkv > 0 && a.nq % a.nkv == 0, "attention: %d query heads do not divide into %d key heads",
+            a.nq, a.nkv);
+  QRT_CHECK(D <= 256, "attention (decode): head size %d is above 256", D);
+  QRT_CHECK(a.page_size > 0 && a.page_size % 8 == 0,
+            "attention (bfloat16): page size %d must be a multiple of 8", a.page_size);
+  QRT_CHECK(a.num_splits >= 1 && a.num_splits <= 65535 && a.nkv <= 65535, "attention: bad split or head count");
+  QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse && counters && num_counters >= a.num_tiles * a.nkv),
+            "attention: split run without scratch or with %d counters for %d", num_counters, a.num_tiles * a.nkv);
+  QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
+  if (a.num_tiles == 0) return 0;
+  dim3 grid(a.num_tiles, a.nkv, a.num_splits), block(64 * DW);
+  const size_t smem = (size_t)(2 * DW * 16 + DW * 16 * D) * sizeof(float);
+  attention_bf16_decode_kernel<<<grid, block, smem, stream>>>(da);
+  QRT_LAUNCH_CHECK("attention_bf16_decode");
+  return 0;
 }
 
 extern "C" int qrt_attention_bf16_head_dim() { return D; }

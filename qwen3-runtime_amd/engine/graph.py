@@ -80,8 +80,7 @@ class DecodeGraph:
                 self.views_dev = self._views()
                 packed.kv_lens = [self.bucket] * self.batch  # launch shapes are those of the bucket
                 self.ctx = runner._context(packed, self.views_dev)
-                self.ctx.scratch["attn_splits"] = runner.ops.choose_splits(
-                    self.batch, self._min_kv_heads(), self.bucket)
+                # the bucket's length, not the batch's, now fixes every launch shape (key splits too)
                 self.cache_views = [
                     None if st.cache is None else runner.cache.view(st.cache, self.ctx.groups, st.writes_cache)
                     for st in runner.model.plan.order

@@ -143,7 +143,7 @@ def build_library(name: str, force: bool = False) -> Path:
     return so
 
 
-def build_all(head_dims=(16, 32, 48, 64, 80, 96, 128, 256), force: bool = True) -> list[Path]:
+def build_all(head_dims=(16, 32, 48, 64, 80, 96, 112, 128, 256), force: bool = True) -> list[Path]:
     """Every library the tests, the smoke run and the measurements load."""
     names = ["core"] + [f"attn_bf16_d{d}" for d in head_dims]
     return [build_library(n, force=force) for n in names]

@@ -347,16 +347,24 @@ class HipOps:
 
     @staticmethod
     def choose_splits(num_tiles: int, nkv: int, max_kv: int) -> int:
-        """How many ways to split the keys so that few long sequences still fill the chip."""
+        """Portions: how many ways to split the keys so that few long sequences still fill the chip."""
         work = num_tiles * nkv
         if max_kv <= 512 or work >= 512:
             return 1
         return max(1, min((max_kv + 255) // 256, (1024 + work - 1) // work, 64))
 
+    @staticmethod
+    def choose_decode_splits(num_tiles: int, nkv: int, max_kv: int) -> int:
+        """Decoding: blocks of four waves; about 512 blocks in all, at least 8 key blocks of 32 each."""
+        work = num_tiles * nkv
+        blocks = (max_kv + 31) // 32
+        return max(1, min((512 + work - 1) // work, blocks // 8, 64))
+
     def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window):
         lib = attention_library(d)
         g = nq // nkv
         max_rows = ctx.max_q_len * g
+        decode = max_rows <= 16 and d <= 256
         waves = 1 if max_rows <= 16 else (2 if max_rows <= 32 else 4)
         key = ("attn_tiles", g, waves)
         plan = ctx.scratch.get(key)
@@ -365,7 +373,9 @@ class HipOps:
             plan = (torch.from_numpy(host).to(q.device), n_tiles)
             ctx.scratch[key] = plan
         tiles, n_tiles = plan
-        splits = ctx.scratch.get("attn_splits") or self.choose_splits(n_tiles, nkv, ctx.max_kv_len)
+        splits = ctx.scratch.get("attn_splits") or (
+            self.choose_decode_splits(n_tiles, nkv, ctx.max_kv_len) if decode
+            else self.choose_splits(n_tiles, nkv, ctx.max_kv_len))
         a = _AttnTileArgs()
         a.q, a.out, a.k_cache, a.v_cache = q.data_ptr(), out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
         a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
@@ -380,7 +390,19 @@ class HipOps:
             part_o = torch.empty((ctx.num_tokens * nq * splits, d), dtype=torch.float32, device=q.device)
             part_lse = torch.empty((ctx.num_tokens * nq * splits,), dtype=torch.float32, device=q.device)
             a.part_o, a.part_lse = part_o.data_ptr(), part_lse.data_ptr()
-        self._check(lib, lib.qrt_attention_bf16(byref(a), c_int(ctx.num_tokens * nq), _stream()))
+        if decode:
+            counters = self._attention_counters(n_tiles * nkv, q.device)
+            self._check(lib, lib.qrt_attention_bf16_decode(byref(a), _ptr(counters), c_int(counters.numel()),
+                                                           _stream()))
+        else:
+            self._check(lib, lib.qrt_attention_bf16(byref(a), c_int(ctx.num_tokens * nq), _stream()))
+
+    def _attention_counters(self, n: int, device) -> torch.Tensor:
+        """Arrival counters of the split merge: zero between launches (the kernel resets them)."""
+        have = getattr(self, "_counters", None)
+        if have is None or have.numel() < n or have.device != device:
+            self._counters = torch.zeros(max(n, 4096), dtype=torch.int32, device=device)
+        return self._counters
 
     # ---- sampling ------------------------------------------------------------------
     def argmax(self, logits):

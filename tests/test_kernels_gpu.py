@@ -274,6 +274,36 @@ def test_paged_attention_splits_agree(ops):
         close(got, want, 2e-2, 2e-2)
 
 
+def test_decode_attention_many_sequences_and_repeated_launches(ops):
+    """The arrival counters of the split merge are left at zero by every launch."""
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(1, 1500, (37,), generator=g).tolist() + [1, 32, 33, 2048]
+    seqs, nq, nkv, d, ps = [(1, n) for n in lens], 8, 2, 128, 16
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, seed=3)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, 0.088)
+    for splits in (5, 1, 16, 3, None):
+        ctx.scratch.pop("attn_splits", None)
+        if splits:
+            ctx.scratch["attn_splits"] = splits
+        got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 0.088, None)
+        close(got, want, 2e-2, 2e-2)
+    assert int(ops._counters.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("seqs,nq,nkv,d,ps", [([(9, 50)], 3, 3, 80, 16), ([(2, 300), (1, 50)], 5, 1, 48, 8),
+                                              ([(7, 90)], 2, 1, 112, 16), ([(40, 90)], 2, 1, 48, 16)])
+def test_attention_repeats_bit_for_bit_at_head_sizes_with_a_16_wide_remainder(ops, seqs, nq, nkv, d, ps):
+    """These head sizes once chained two MFMA shapes, whose results then differed from run to run."""
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, 1 / math.sqrt(d))
+    first = ops.paged_attention(q, cache, ctx, nq, nkv, d, 1 / math.sqrt(d), None)
+    close(first, want, 2e-2, 2e-2)
+    for _ in range(100):
+        assert torch.equal(ops.paged_attention(q, cache, ctx, nq, nkv, d, 1 / math.sqrt(d), None), first)
+
+
 def test_attention_far_key_stands_out(ops):
     """One early key is made to dominate; the context must equal its value."""
     for dtype in (torch.float32, torch.bfloat16):
