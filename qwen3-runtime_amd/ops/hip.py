@@ -355,10 +355,10 @@ class HipOps:
 
     @staticmethod
     def choose_decode_splits(num_tiles: int, nkv: int, max_kv: int) -> int:
-        """Decoding: blocks of four waves; about 512 blocks in all, at least 8 key blocks of 32 each."""
+        """Decoding: blocks of four waves; about 256 blocks in all, at least 8 key blocks of 32 each."""
         work = num_tiles * nkv
         blocks = (max_kv + 31) // 32
-        return max(1, min((512 + work - 1) // work, blocks // 8, 64))
+        return max(1, min((256 + work - 1) // work, blocks // 8, 64))
 
     def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window):
         lib = attention_library(d)
@@ -391,18 +391,9 @@ class HipOps:
             part_lse = torch.empty((ctx.num_tokens * nq * splits,), dtype=torch.float32, device=q.device)
             a.part_o, a.part_lse = part_o.data_ptr(), part_lse.data_ptr()
         if decode:
-            counters = self._attention_counters(n_tiles * nkv, q.device)
-            self._check(lib, lib.qrt_attention_bf16_decode(byref(a), _ptr(counters), c_int(counters.numel()),
-                                                           _stream()))
+            self._check(lib, lib.qrt_attention_bf16_decode(byref(a), c_int(ctx.num_tokens * nq), _stream()))
         else:
             self._check(lib, lib.qrt_attention_bf16(byref(a), c_int(ctx.num_tokens * nq), _stream()))
-
-    def _attention_counters(self, n: int, device) -> torch.Tensor:
-        """Arrival counters of the split merge: zero between launches (the kernel resets them)."""
-        have = getattr(self, "_counters", None)
-        if have is None or have.numel() < n or have.device != device:
-            self._counters = torch.zeros(max(n, 4096), dtype=torch.int32, device=device)
-        return self._counters
 
     # ---- sampling ------------------------------------------------------------------
     def argmax(self, logits):

