@@ -96,6 +96,7 @@ struct SampleArgs {
   int* out_token;           // [R]
   float* out_logprob;       // [R]
   int rows, vocab;
+  int write_work;           // also keep the processed logits of greedy rows
 };
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
@@ -109,9 +110,16 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   const float* fp = a.fparams + (size_t)sl * 8;
   const float temp = fp[0], topp = fp[1], minp = fp[2], rep = fp[3], pres = fp[4], freq = fp[5];
 
-  // penalties (reference: qwen3_runtime/sampling.py:63-71)
+  // one pass: penalties (reference: qwen3_runtime/sampling.py:63-71) and temperature give the
+  // processed value; alongside, a running maximum, the first index that reaches it, and the sum
+  // of exp(value - maximum)
   const bool pen = a.counts && (rep != 1.0f || pres != 0.0f || freq != 0.0f);
   const int* cnt = pen ? a.counts + (size_t)sl * V : nullptr;
+  const bool greedy = temp <= 0.f;
+  const bool keep = !greedy || a.write_work;
+  float m = -INFINITY, ssum = 0.f;
+  int bi = 0x7fffffff;
+#pragma unroll 4
   for (int i = tid; i < V; i += blockDim.x) {
     float v = lg[i];
     if (cnt) {
@@ -122,24 +130,59 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
         v -= freq * (float)c;
       }
     }
-    if (temp > 0.f) v = v / temp;
-    x[i] = v;
+    if (!greedy) v = v / temp;
+    if (keep) x[i] = v;
+    if (v > m) {
+      ssum = ssum * expf(m - v) + 1.0f;  // m = -inf at first: exp(-inf) = 0
+      m = v;
+      bi = i;
+    } else if (v == v) {
+      ssum += expf(v - m);
+    }
   }
-  __syncthreads();
+  // merge over the wave, then over the block: the larger maximum wins, ties go to the lower index
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float om = __shfl_xor(m, o, 64), os = __shfl_xor(ssum, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    const float mm = fmaxf(m, om);
+    const float f1 = m == -INFINITY ? 0.f : expf(m - mm), f2 = om == -INFINITY ? 0.f : expf(om - mm);
+    ssum = ssum * f1 + os * f2;
+    if (om > m || (om == m && oi < bi)) bi = oi;
+    m = mm;
+  }
+  {
+    const int lane = tid & 63, wave = tid >> 6, nw = (blockDim.x + 63) >> 6;
+    if (lane == 0) { red[wave] = m; part[wave] = ssum; redi[wave] = bi; }
+    __syncthreads();
+    if (tid == 0) {
+      float mm = red[0], ss = part[0];
+      int ii = redi[0];
+      for (int w = 1; w < nw; ++w) {
+        const float om = red[w], os = part[w];
+        const int oi = redi[w];
+        const float nm = fmaxf(mm, om);
+        const float f1 = mm == -INFINITY ? 0.f : expf(mm - nm), f2 = om == -INFINITY ? 0.f : expf(om - nm);
+        ss = ss * f1 + os * f2;
+        if (om > mm || (om == mm && oi < ii)) ii = oi;
+        mm = nm;
+      }
+      if (ii == 0x7fffffff) ii = 0;  // a row of NaNs
+      red[24] = mm; red[25] = ss; redi[24] = ii;
+    }
+    __syncthreads();
+  }
+  const float mx = red[24];
+  const int best = redi[24];
 
-  float mx;
-  int best = block_argmax(x, V, red, redi, &mx);
-
-  if (temp <= 0.f) {  // greedy; logprob = log_softmax(processed)[tok]
-    float s = 0.f;
-    for (int i = tid; i < V; i += blockDim.x) s += expf(x[i] - mx);
-    s = block_sum(s, red);
+  if (greedy) {  // logprob = log_softmax(processed)[tok] = -log(sum of exp(x - max))
     if (tid == 0) {
       a.out_token[r] = best;
-      a.out_logprob[r] = -logf(s);
+      a.out_logprob[r] = -logf(red[25]);
     }
     return;
   }
+  __syncthreads();
 
   // min_p: drop ids with p < min_p * p_max  <=>  x < max + log(min_p)
   if (minp > 0.f) {

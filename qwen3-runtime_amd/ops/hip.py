@@ -71,6 +71,7 @@ class _SampleArgs(Structure):
         ("logits", c_void_p), ("work", c_void_p), ("counts", c_void_p), ("slot", c_void_p),
         ("fparams", c_void_p), ("iparams", c_void_p), ("seeds", c_void_p),
         ("out_token", c_void_p), ("out_logprob", c_void_p), ("rows", c_int), ("vocab", c_int),
+        ("write_work", c_int),
     ]
 
 
@@ -128,7 +129,7 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> torch.Tensor:
 
 class HipOps:
     # bfloat16 products with more rows than this go to the vendor BLAS
-    blas_min_rows = 128
+    own_max_rows = 16
 
     def __init__(self):
         self.lib = core_library()
@@ -190,7 +191,11 @@ class HipOps:
             return out if (out_f32 or x.dtype == torch.float32) else out.to(x.dtype)
         if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
             raise OpsError(f"linear: no product of {x.dtype} activations with {w.dtype} weights")
-        if m >= self.blas_min_rows and not out_f32:
+        if m > self.own_max_rows:
+            # measured at the 4B shapes: from about 32 rows on the vendor library streams the
+            # weights faster than the few-row kernel; both accumulate in float32
+            if out_f32:
+                return torch.mm(x, w.t(), out_dtype=torch.float32)
             return torch.matmul(x, w.t())
         out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
         self._check(self.lib, self.lib.qrt_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), F32 if out_f32 else BF16,
@@ -198,7 +203,7 @@ class HipOps:
         return out
 
     # rows up to which the gated activation is fused into the product before it
-    fused_gate_max_rows = 64
+    fused_gate_max_rows = 16
 
     def gated_linear(self, x, w_gate_up):
         """``swiglu(linear(x, w_gate_up))`` with ``w_gate_up`` [2I, K], gate rows first. With few
@@ -403,7 +408,7 @@ class HipOps:
         self._check(self.lib, self.lib.qrt_argmax(_ptr(logits), _ptr(out), c_int(r), c_int(v), _stream()))
         return out
 
-    def sample(self, logits, slot, fparams, iparams, seeds, counts=None):
+    def sample(self, logits, slot, fparams, iparams, seeds, counts=None, keep_processed=False):
         """One token per row of ``logits``. Options are read from the row's state slot:
         ``fparams[slot]`` = temperature, top_p, min_p, repetition, presence, frequency;
         ``iparams[slot]`` = top_k; ``seeds[slot]`` = seed, index of the next draw (advanced
@@ -424,6 +429,7 @@ class HipOps:
         a.logits, a.work, a.counts, a.slot = logits.data_ptr(), work.data_ptr(), _addr(counts), slot.data_ptr()
         a.fparams, a.iparams, a.seeds = fparams.data_ptr(), iparams.data_ptr(), seeds.data_ptr()
         a.out_token, a.out_logprob, a.rows, a.vocab = tok.data_ptr(), lp.data_ptr(), r, v
+        a.write_work = 1 if keep_processed else 0  # greedy rows skip the write unless asked
         self._check(self.lib, self.lib.qrt_sample(byref(a), _stream()))
         return tok, lp, work
 

@@ -54,9 +54,11 @@ class Sampler:
             toks = torch.tensor([int(b[1]) for b in bias], dtype=torch.int32, device=self.device)
             vals = torch.tensor([float(b[2]) for b in bias], dtype=torch.float32, device=self.device)
             self.ops.add_bias(logits, rows, toks, vals)
-        tok, lp, work = self.ops.sample(logits, slot_rows, self.fparams, self.iparams, self.seeds, self.counts)
         forced = [r.next_forced_token() for r in reqs]
-        if any(f is not None for f in forced):
+        any_forced = any(f is not None for f in forced)
+        tok, lp, work = self.ops.sample(logits, slot_rows, self.fparams, self.iparams, self.seeds, self.counts,
+                                        keep_processed=any_forced)
+        if any_forced:
             # teacher forcing: the given id, scored under the processed logits
             # (reference: qwen3_runtime/sampling.py:319-325)
             logp = torch.log_softmax(work, dim=-1)

@@ -100,8 +100,9 @@ def test_gemm_bf16(ops, m, n, k, out_f32):
 
 @pytest.mark.parametrize("m,i,k", [(1, 9728, 2560), (8, 288, 96), (33, 100, 64), (64, 272, 96), (70, 64, 64),
                                    (5, 64, 48), (16, 1000, 128)])
-def test_gated_linear(ops, m, i, k):
+def test_gated_linear(ops, m, i, k, monkeypatch):
     """The fused form (few rows) and the two-kernel form agree with the plain one."""
+    monkeypatch.setattr(ops, "fused_gate_max_rows", 64)
     for dtype in (torch.bfloat16, torch.float32):
         x, w = rnd(m, k, dtype=dtype, seed=3), rnd(2 * i, k, dtype=dtype, seed=4, scale=0.05)
         gu = x.double() @ w.double().T
@@ -114,12 +115,18 @@ def test_gated_linear(ops, m, i, k):
         close(got, want, tol, tol)
 
 
+@pytest.mark.parametrize("own_max_rows", [16, 1 << 30])
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 40, 64])
 @pytest.mark.parametrize("n,k", [(6144, 2560), (2560, 4096), (1000, 9728), (272, 96)])
-def test_gemm_bf16_few_rows_at_model_sizes(ops, m, n, k):
+def test_gemm_bf16_few_rows_at_model_sizes(ops, m, n, k, own_max_rows, monkeypatch):
+    """Above ``own_max_rows`` rows the vendor library takes over; the library's own kernels for up
+    to 64 rows stay correct behind it."""
+    monkeypatch.setattr(ops, "own_max_rows", own_max_rows)
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.02)
     want = x.double() @ w.double().T
-    close(ops.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
+    got = ops.linear(x, w, out_f32=True)
+    assert got.dtype == torch.float32
+    close(got, want, 2e-3, 2e-3)
     close(ops.linear(x, w), want, 3e-2, 3e-2)
 
 
