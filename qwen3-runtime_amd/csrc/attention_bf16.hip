@@ -61,6 +61,7 @@ struct AttnTileArgs {
   float* part_lse;        // [T, nq, num_splits]      base-2 log of the split's sum, -inf if empty
   int table_width, num_tiles, nq, nkv, page_size, window, num_splits, waves;
   float scale_log2;
+  int row_tiles;  // tiles of 16 rows per wave (general kernel): 1, 2 or 4
 };
 
 constexpr int D = QRT_HEAD_DIM;
@@ -68,7 +69,13 @@ constexpr int KFULL = D / 32;        // 32-wide steps of the first product
 constexpr bool KTAIL = (D % 32) != 0;  // one 16-wide step more
 constexpr int DB = D / 16;           // 16-wide blocks of the head dimension
 
-__global__ __launch_bounds__(256) void attention_bf16_kernel(AttnTileArgs a) {
+// General kernel (prompt portions and mixed batches). A wave owns RT tiles of 16
+// rows each, 16 * RT consecutive rows of the sequence's row matrix; a block is
+// four waves, 64 * RT rows. The keys and values of a block of 32 keys are read
+// once into registers and multiplied with all RT tiles, which divides the
+// operand traffic per MFMA by RT.
+template <int RT>
+__global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(AttnTileArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
   const int seq = a.tile_seq[blockIdx.x];
@@ -78,28 +85,35 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnTileArgs a) {
   const int q_len = a.cu_q[seq + 1] - q_begin;
   const int kv_len = a.kv_lens[seq];
   const int n_rows = q_len * g;
-  const int row0 = a.tile_row0[blockIdx.x] + 16 * wave;
+  const int row0 = a.tile_row0[blockIdx.x] + 16 * RT * wave;
   if (row0 >= n_rows) return;
   const int first_pos = kv_len - q_len;
-  const int my_row = row0 + r16;
-  const bool row_valid = my_row < n_rows;
-  const int row_c = row_valid ? my_row : n_rows - 1;
-  const int tok = row_c / g, hg = row_c - tok * g;
-  const int qpos = first_pos + tok;
-  const int head = kvh * g + hg;
   const int ps = a.page_size;
   const int* table = a.block_table + (size_t)seq * a.table_width;
 
-  // Q as B operands, kept for the whole loop
-  const bf16_t* qp = a.q + ((size_t)(q_begin + tok) * a.nq + head) * D;
-  bf16x8_t qreg[KFULL > 0 ? KFULL : 1];
+  // per tile: this lane's row, its token's position, and Q as B operands kept for the whole loop
+  bool row_valid[RT];
+  int qpos[RT];
+  size_t row_index[RT];
+  bf16x8_t qreg[RT][KFULL > 0 ? KFULL : 1];
+  bf16x8_t qtail[RT];
 #pragma unroll
-  for (int i = 0; i < KFULL; ++i) qreg[i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
-  bf16x8_t qtail = load_tail(qp, 2);  // zeros
-  if (KTAIL) qtail = load_tail(qp + 32 * KFULL, quad);
+  for (int t = 0; t < RT; ++t) {
+    const int my_row = row0 + 16 * t + r16;
+    row_valid[t] = my_row < n_rows;
+    const int row_c = row_valid[t] ? my_row : n_rows - 1;
+    const int tok = row_c / g, hg = row_c - tok * g;
+    qpos[t] = first_pos + tok;
+    row_index[t] = (size_t)(q_begin + tok) * a.nq + kvh * g + hg;
+    const bf16_t* qp = a.q + row_index[t] * D;
+#pragma unroll
+    for (int i = 0; i < KFULL; ++i) qreg[t][i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
+    qtail[t] = load_tail(qp, 2);  // zeros
+    if (KTAIL) qtail[t] = load_tail(qp + 32 * KFULL, quad);
+  }
 
   // keys this wave may need: [lo, pos_max]
-  const int row_last = min(row0 + 15, n_rows - 1);
+  const int row_last = min(row0 + 16 * RT - 1, n_rows - 1);
   const int pos_min = first_pos + row0 / g, pos_max = first_pos + row_last / g;
   const int lo = a.window > 0 ? max(0, pos_min - a.window + 1) : 0;
   const int blk_begin = lo >> 5, blk_end = (pos_max >> 5) + 1;
@@ -107,99 +121,115 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnTileArgs a) {
   const int b0 = blk_begin + split * per;
   const int b1 = min(blk_end, b0 + per);
 
-  f32x4_t o[DB];
+  f32x4_t o[RT][DB];
+  float m[RT], l[RT];
 #pragma unroll
-  for (int i = 0; i < DB; ++i) o[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+  for (int t = 0; t < RT; ++t) {
+    m[t] = -INFINITY;
+    l[t] = 0.f;
+#pragma unroll
+    for (int i = 0; i < DB; ++i) o[t][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  }
 
   for (int b = b0; b < b1; ++b) {
     const int base = b << 5;
-    f32x4_t s[2];
+    // keys of the block as A operands: row 4 quad' + r of sub-block kb holds key 8 quad' + 4 kb + r
+    bf16x8_t kk[2][KFULL > 0 ? KFULL : 1], kt[2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       int kidx = base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3);
       kidx = min(max(kidx, lo), pos_max);  // stay inside pages this sequence holds; masked below
       const int page = table[kidx / ps];
       const bf16_t* kp = a.k_cache + (((size_t)page * a.nkv + kvh) * ps + (kidx % ps)) * D;
-      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < KFULL; ++i) {
-        const bf16x8_t kk = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk, qreg[i], acc, 0, 0, 0);
-      }
-      if (KTAIL) {
-        const bf16x8_t kk = load_tail(kp + 32 * KFULL, quad);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk, qtail, acc, 0, 0, 0);
-      }
-      s[kb] = acc;
+      for (int i = 0; i < KFULL; ++i) kk[kb][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
+      if (KTAIL) kt[kb] = load_tail(kp + 32 * KFULL, quad);
     }
-    // this lane: row r16, keys base + 8 quad + 4 kb + r
-    float p[8];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int key = base + 8 * quad + e;
-      const bool vis = row_valid && key <= qpos && (a.window == 0 || key > qpos - a.window);
-      p[e] = vis ? s[e >> 2][e & 3] * a.scale_log2 : -INFINITY;
-      mx = fmaxf(mx, p[e]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = exp2f(m - m_use);
-    float psum = 0.f;
-    bf16x8_t pb;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float pe = exp2f(p[e] - m_use);
-      psum += pe;
-      pb[e] = (bf16_t)pe;
-    }
-    l = l * corr + psum;
-    m = m_new;
-#pragma unroll
-    for (int i = 0; i < DB; ++i) o[i] *= corr;
-
     // values: 8 consecutive keys base + 8 quad .. + 7 of head element 16 i + r16
     const int kv0 = base + 8 * quad;
     const bool vload = kv0 <= pos_max && kv0 + 7 >= lo;
     const int vpage = vload ? table[kv0 / ps] : 0;
     const bf16_t* vp = a.v_cache + (((size_t)vpage * a.nkv + kvh) * D + r16) * ps + (kv0 % ps);
+    bf16x8_t vv[DB];
 #pragma unroll
     for (int i = 0; i < DB; ++i) {
-      bf16x8_t vv;
-      if (vload) vv = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
+      if (vload) vv[i] = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
       else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) vv[e] = (bf16_t)0.0f;
+        for (int e = 0; e < 8; ++e) vv[i][e] = (bf16_t)0.0f;
       }
-      o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, pb, o[i], 0, 0, 0);
+    }
+
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      f32x4_t s[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < KFULL; ++i)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk[kb][i], qreg[t][i], acc, 0, 0, 0);
+        if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[kb], qtail[t], acc, 0, 0, 0);
+        s[kb] = acc;
+      }
+      // this lane: row r16 of tile t, keys base + 8 quad + 4 kb + r
+      float p[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = base + 8 * quad + e;
+        const bool vis = row_valid[t] && key <= qpos[t] && (a.window == 0 || key > qpos[t] - a.window);
+        p[e] = vis ? s[e >> 2][e & 3] * a.scale_log2 : -INFINITY;
+        mx = fmaxf(mx, p[e]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[t], mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float corr = exp2f(m[t] - m_use);
+      float psum = 0.f;
+      bf16x8_t pb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float pe = exp2f(p[e] - m_use);
+        psum += pe;
+        pb[e] = (bf16_t)pe;
+      }
+      l[t] = l[t] * corr + psum;
+      m[t] = m_new;
+#pragma unroll
+      for (int i = 0; i < DB; ++i) {
+        o[t][i] *= corr;
+        o[t][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[i], pb, o[t][i], 0, 0, 0);
+      }
     }
   }
 
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  if (!row_valid) return;
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
-  const size_t row_index = (size_t)(q_begin + tok) * a.nq + head;
-  if (a.num_splits == 1) {
-    bf16_t* op = a.out + row_index * D;
 #pragma unroll
-    for (int i = 0; i < DB; ++i) {
-      bf16x4_t w;
+  for (int t = 0; t < RT; ++t) {
+    float lt = l[t];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    if (!row_valid[t]) continue;
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    if (a.num_splits == 1) {
+      bf16_t* op = a.out + row_index[t] * D;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) w[r] = (bf16_t)(o[i][r] * inv);
-      *(bf16x4_t*)(op + 16 * i + 4 * quad) = w;
+      for (int i = 0; i < DB; ++i) {
+        bf16x4_t w;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) w[r] = (bf16_t)(o[t][i][r] * inv);
+        *(bf16x4_t*)(op + 16 * i + 4 * quad) = w;
+      }
+    } else {
+      float* op = a.part_o + (row_index[t] * a.num_splits + split) * D;
+#pragma unroll
+      for (int i = 0; i < DB; ++i) {
+        f32x4_t w = o[t][i] * inv;
+        *(f32x4_t*)(op + 16 * i + 4 * quad) = w;
+      }
+      if (quad == 0) a.part_lse[row_index[t] * a.num_splits + split] = lt > 0.f ? m[t] + log2f(lt) : -INFINITY;
     }
-  } else {
-    float* op = a.part_o + (row_index * a.num_splits + split) * D;
-#pragma unroll
-    for (int i = 0; i < DB; ++i) {
-      f32x4_t w = o[i] * inv;
-      *(f32x4_t*)(op + 16 * i + 4 * quad) = w;
-    }
-    if (quad == 0) a.part_lse[row_index * a.num_splits + split] = l > 0.f ? m + log2f(l) : -INFINITY;
   }
 }
 
@@ -476,7 +506,10 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
   if (a.num_tiles == 0) return 0;
   dim3 grid(a.num_tiles, a.nkv, a.num_splits), block(64 * a.waves);
-  attention_bf16_kernel<<<grid, block, 0, stream>>>(a);
+  if (a.row_tiles == 1) attention_bf16_kernel<1><<<grid, block, 0, stream>>>(a);
+  else if (a.row_tiles == 2) attention_bf16_kernel<2><<<grid, block, 0, stream>>>(a);
+  else if (a.row_tiles == 4 && D <= 128) attention_bf16_kernel<4><<<grid, block, 0, stream>>>(a);
+  else return qrt_fail("attention: %d row tiles per wave at head size %d is not built", a.row_tiles, D);
   QRT_LAUNCH_CHECK("attention_bf16");
   if (a.num_splits > 1) {
     attention_merge_kernel<<<dim3(num_rows_total), dim3(D >= 64 ? 64 : 32), 0, stream>>>(a.part_o, a.part_lse, a.out,

@@ -62,7 +62,7 @@ class _AttnTileArgs(Structure):
         ("tile_seq", c_void_p), ("tile_row0", c_void_p), ("part_o", c_void_p), ("part_lse", c_void_p),
         ("table_width", c_int), ("num_tiles", c_int), ("nq", c_int), ("nkv", c_int),
         ("page_size", c_int), ("window", c_int), ("num_splits", c_int), ("waves", c_int),
-        ("scale_log2", c_float),
+        ("scale_log2", c_float), ("row_tiles", c_int),
     ]
 
 
@@ -130,6 +130,8 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> torch.Tensor:
 class HipOps:
     # bfloat16 products with more rows than this go to the vendor BLAS
     own_max_rows = 16
+    # tiles of 16 rows per wave in the attention kernel for long portions (1, 2 or 4)
+    prefill_row_tiles = 2
 
     def __init__(self):
         self.lib = core_library()
@@ -340,14 +342,20 @@ class HipOps:
         return out
 
     @staticmethod
-    def plan_tiles(q_lens, group_size: int, waves: int):
-        """Work list of the MFMA attention kernel: (sequence, first row) per tile of 16*waves rows."""
-        rows_per_tile = 16 * waves
-        seqs, row0 = [], []
-        for s, n in enumerate(q_lens):
+    def plan_tiles(q_lens, kv_lens, group_size: int, rows_per_tile: int):
+        """Work list of the MFMA attention kernels: (sequence, first row) per tile of rows.
+
+        Tiles that see the most keys come first: blocks that start late are then the short ones,
+        and the chip stays full until the end although causal tiles differ in length."""
+        items = []
+        for s, (n, kv) in enumerate(zip(q_lens, kv_lens)):
+            first = kv - n
             for r in range(0, n * group_size, rows_per_tile):
-                seqs.append(s)
-                row0.append(r)
+                last_tok = min(n * group_size, r + rows_per_tile) - 1
+                items.append((-(first + last_tok // group_size), s, r))
+        items.sort()
+        seqs = [s for _, s, _ in items]
+        row0 = [r for _, _, r in items]
         return np.asarray(seqs + row0, dtype=np.int32), len(seqs)
 
     @staticmethod
@@ -371,10 +379,12 @@ class HipOps:
         max_rows = ctx.max_q_len * g
         decode = max_rows <= 16 and d <= 256
         waves = 1 if max_rows <= 16 else (2 if max_rows <= 32 else 4)
-        key = ("attn_tiles", g, waves)
+        # long portions: several row tiles per wave, so that loaded keys and values serve more rows
+        row_tiles = 1 if max_rows <= 64 else (self.prefill_row_tiles if d <= 128 else min(2, self.prefill_row_tiles))
+        key = ("attn_tiles", g, waves, row_tiles)
         plan = ctx.scratch.get(key)
         if plan is None:
-            host, n_tiles = self.plan_tiles(ctx.q_lens_host, g, waves)
+            host, n_tiles = self.plan_tiles(ctx.q_lens_host, ctx.kv_lens_host, g, 16 * waves * row_tiles)
             plan = (torch.from_numpy(host).to(q.device), n_tiles)
             ctx.scratch[key] = plan
         tiles, n_tiles = plan
@@ -389,7 +399,7 @@ class HipOps:
         a.tile_seq = tiles.data_ptr()
         a.tile_row0 = tiles.data_ptr() + 4 * n_tiles
         a.num_tiles, a.nq, a.nkv, a.page_size, a.window = n_tiles, nq, nkv, cache.group.page_size, window
-        a.num_splits, a.waves = splits, waves
+        a.num_splits, a.waves, a.row_tiles = splits, waves, row_tiles
         a.scale_log2 = scale * math.log2(math.e)
         if splits > 1:
             part_o = torch.empty((ctx.num_tokens * nq * splits, d), dtype=torch.float32, device=q.device)
