@@ -83,34 +83,52 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
 }
 
 // ------------------------------------------------------------------ SwiGLU
-// out[t, i] = silu(gu[t, i]) * gu[t, I + i],  silu(x) = x / (1 + exp(-x))
-template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i],  silu(x) = x / (1 + exp(-x)), in float32.
+// VEC elements per thread and access: 8 for bfloat16 rows whose halves start on 16 bytes.
+template <typename T, int VEC>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total_vec) {
+  typedef T vec_t __attribute__((ext_vector_type(VEC)));
+  const int per_row = inter / VEC;
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (; idx < total; idx += stride) {
-    const size_t t = idx / inter;
-    const int i = (int)(idx - t * inter);
-    const float g = to_f32<T>(gu[t * 2 * inter + i]);
-    const float u = to_f32<T>(gu[t * 2 * inter + inter + i]);
-    out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+  for (; idx < total_vec; idx += stride) {
+    const size_t t = idx / per_row;
+    const int i = (int)(idx - t * per_row) * VEC;
+    const vec_t g = *(const vec_t*)(gu + t * 2 * inter + i);
+    const vec_t u = *(const vec_t*)(gu + t * 2 * inter + inter + i);
+    vec_t o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float gf = to_f32<T>(g[e]);
+      o[e] = from_f32<T>(gf / (1.0f + expf(-gf)) * to_f32<T>(u[e]));
+    }
+    *(vec_t*)(out + t * inter + i) = o;
   }
+}
+
+template <typename T, int VEC>
+static void swiglu_launch(const void* gate_up, void* out, int num_tokens, int inter, hipStream_t stream) {
+  const size_t total = (size_t)num_tokens * (inter / VEC);
+  const int block = 256;
+  size_t blocks = (total + block - 1) / block;
+  if (blocks > 16384) blocks = 16384;
+  swiglu_kernel<T, VEC><<<dim3((unsigned)blocks), block, 0, stream>>>((const T*)gate_up, (T*)out, inter, total);
 }
 
 extern "C" int qrt_swiglu(const void* gate_up, void* out, int dtype, int num_tokens, int inter,
                           hipStream_t stream) {
   QRT_CHECK(num_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", num_tokens, inter);
-  const size_t total = (size_t)num_tokens * inter;
-  if (total == 0) return 0;
-  const int block = 256;
-  size_t blocks = (total + block - 1) / block;
-  if (blocks > 65536) blocks = 65536;
-  if (dtype == QRT_F32)
-    swiglu_kernel<float><<<dim3((unsigned)blocks), block, 0, stream>>>((const float*)gate_up, (float*)out, inter, total);
-  else if (dtype == QRT_BF16)
-    swiglu_kernel<bf16_t><<<dim3((unsigned)blocks), block, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, total);
-  else
+  if ((size_t)num_tokens * inter == 0) return 0;
+  const bool aligned = ((uintptr_t)gate_up % 16 == 0) && ((uintptr_t)out % 16 == 0);
+  if (dtype == QRT_F32) {
+    if (aligned && inter % 4 == 0) swiglu_launch<float, 4>(gate_up, out, num_tokens, inter, stream);
+    else swiglu_launch<float, 1>(gate_up, out, num_tokens, inter, stream);
+  } else if (dtype == QRT_BF16) {
+    if (aligned && inter % 8 == 0) swiglu_launch<bf16_t, 8>(gate_up, out, num_tokens, inter, stream);
+    else swiglu_launch<bf16_t, 1>(gate_up, out, num_tokens, inter, stream);
+  } else {
     return qrt_fail("swiglu: unknown dtype %d", dtype);
+  }
   QRT_LAUNCH_CHECK("swiglu");
   return 0;
 }
