@@ -41,6 +41,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill measurement")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="measure only the 2,048-token prefill (for profiling); prints a reduced line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine is single-GPU)")
@@ -59,7 +61,7 @@ def main() -> int:
     cfg = cfg_full if args.layers is None else dataclasses.replace(cfg_full, num_hidden_layers=args.layers)
     steps, warmup = args.steps, args.warmup
     page = 16
-    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    max_batch = args.batch if (args.no_points or args.prefill_only) else max(args.batch, 64)
     per_req_tokens = args.prompt_len + steps + warmup + max_batch + 10
     pages = max_batch * (-(-per_req_tokens // page) + 1)
     t0 = time.time()
@@ -96,23 +98,8 @@ def main() -> int:
             engine.finish_request(r.request_id)
         return dt, kv_tokens
 
-    dt, kv_tokens = decode_run(args.batch, steps, warmup)
-    ms_per_step = dt / steps * 1e3
-    value = args.batch * steps / dt
-    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.kv_width * bytes_el
-    # every weight the step uses, once: the tied table is read once, as the head
-    head_bytes = cfg.vocab_size * cfg.hidden_size * bytes_el
-    step_weight_bytes = engine.loaded.weight_bytes if cfg.tie_word_embeddings else engine.loaded.weight_bytes - head_bytes
-    step_bytes = step_weight_bytes + kv_tokens * kv_bytes_per_token
-    achieved = step_bytes / (dt / steps) / 1e9
-
-    points, prefill = {}, None
-    if not args.no_points:
-        for b in (1, 64):
-            k = min(steps, 64)
-            d, _ = decode_run(b, k, min(warmup, 8))
-            points[f"decode_b{b}"] = round(b * k / d, 1)
-        # prefill: one 2,048-token prompt through the step function, logits at its last token
+    def prefill_run():
+        """One 2,048-token prompt through the step function, logits at its last token."""
         tokens = 2048
         ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=gen).tolist()
         times = []
@@ -132,8 +119,30 @@ def main() -> int:
         attn = 2 * cfg.q_width * tokens * tokens * cfg.num_hidden_layers
         head = 2 * cfg.vocab_size * cfg.hidden_size
         peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
-        prefill = {"value": round(tokens / pt, 1), "tokens": tokens, "ms": round(pt * 1e3, 3),
-                   "frac": round((lin + attn + head) / pt / peak, 4)}
+        return {"value": round(tokens / pt, 1), "tokens": tokens, "ms": round(pt * 1e3, 3),
+                "frac": round((lin + attn + head) / pt / peak, 4)}
+
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tok/s, one 2,048-token prompt", "prefill": prefill_run()}), flush=True)
+        return 0
+
+    dt, kv_tokens = decode_run(args.batch, steps, warmup)
+    ms_per_step = dt / steps * 1e3
+    value = args.batch * steps / dt
+    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.kv_width * bytes_el
+    # every weight the step uses, once: the tied table is read once, as the head
+    head_bytes = cfg.vocab_size * cfg.hidden_size * bytes_el
+    step_weight_bytes = engine.loaded.weight_bytes if cfg.tie_word_embeddings else engine.loaded.weight_bytes - head_bytes
+    step_bytes = step_weight_bytes + kv_tokens * kv_bytes_per_token
+    achieved = step_bytes / (dt / steps) / 1e9
+
+    points, prefill = {}, None
+    if not args.no_points:
+        for b in (1, 64):
+            k = min(steps, 64)
+            d, _ = decode_run(b, k, min(warmup, 8))
+            points[f"decode_b{b}"] = round(b * k / d, 1)
+        prefill = prefill_run()
 
     line = {
         "metric": "decode tok/s at batch 8 (Qwen3-4B shape, 2,048-token prompts)",
