@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 // GATED: W holds 2N rows, gate rows then up rows; the block owns matching
 // tiles of both and writes silu(gate) * up, so the gated feed-forward's
 // intermediate [M, 2N] never reaches memory.
-template <int MB, int NW, int NT, int U, bool GATED, typename TO>
+template <int MB, int NW, int NT, int U, bool GATED, bool TILED, typename TO>
 __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A,
                                                                     const bf16_t* __restrict__ W,
                                                                     TO* __restrict__ C, int M, int N, int K) {
@@ -111,11 +111,20 @@ __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t*
   const int r16 = lane & 15, quad = lane >> 4;
   const int n0 = blockIdx.x * 16 * NT;
   const bf16_t* wrow[WT];
+  // TILED: W is stored tile by tile, [row tile of 16][k-step of 32][lane][8 elements], each
+  // (tile, step) being exactly the 1 KB a wave loads at once; N is then a multiple of 16
+  constexpr int WSTEP = TILED ? 512 : 32;  // elements between consecutive k-steps of a lane
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int n = min(n0 + 16 * t + r16, N - 1);
-    wrow[t] = W + (size_t)n * K + 8 * quad;
-    if (GATED) wrow[NT + t] = W + (size_t)(N + n) * K + 8 * quad;
+    if (TILED) {
+      const int tile = min(n0 / 16 + t, N / 16 - 1);
+      wrow[t] = W + (size_t)tile * 16 * K + 8 * lane;
+      if (GATED) wrow[NT + t] = W + (size_t)(N / 16 + tile) * 16 * K + 8 * lane;
+    } else {
+      const int n = min(n0 + 16 * t + r16, N - 1);
+      wrow[t] = W + (size_t)n * K + 8 * quad;
+      if (GATED) wrow[NT + t] = W + (size_t)(N + n) * K + 8 * quad;
+    }
   }
   const bf16_t* arow[MB];
   bool avalid[MB];
@@ -142,7 +151,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t*
       const int s = s0 + u * NW;
       if (s < steps) {  // uniform over the wave
 #pragma unroll
-        for (int t = 0; t < WT; ++t) w[u][t] = *(const bf16x8_t*)(wrow[t] + (s << 5));
+        for (int t = 0; t < WT; ++t) w[u][t] = *(const bf16x8_t*)(wrow[t] + (size_t)s * WSTEP);
 #pragma unroll
         for (int b = 0; b < MB; ++b) a[u][b] = avalid[b] ? *(const bf16x8_t*)(arow[b] + (s << 5)) : zero;
       }
@@ -196,15 +205,15 @@ __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t*
   }
 }
 
-template <int MB, int NW, int NT, int U, bool GATED>
+template <int MB, int NW, int NT, int U, bool GATED, bool TILED = false>
 static int launch_skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K,
                          hipStream_t stream) {
   dim3 grid((N + 16 * NT - 1) / (16 * NT)), block(64 * NW);
   const size_t smem = (size_t)NW * (GATED ? 2 : 1) * NT * MB * 4 * 64 * sizeof(float);
   if (out_dtype == QRT_BF16)
-    gemm_bf16_skinny_kernel<MB, NW, NT, U, GATED, bf16_t><<<grid, block, smem, stream>>>(a, w, (bf16_t*)c, M, N, K);
+    gemm_bf16_skinny_kernel<MB, NW, NT, U, GATED, TILED, bf16_t><<<grid, block, smem, stream>>>(a, w, (bf16_t*)c, M, N, K);
   else if (out_dtype == QRT_F32)
-    gemm_bf16_skinny_kernel<MB, NW, NT, U, GATED, float><<<grid, block, smem, stream>>>(a, w, (float*)c, M, N, K);
+    gemm_bf16_skinny_kernel<MB, NW, NT, U, GATED, TILED, float><<<grid, block, smem, stream>>>(a, w, (float*)c, M, N, K);
   else
     return qrt_fail("gemm_bf16: unknown output dtype %d", out_dtype);
   QRT_LAUNCH_CHECK("gemm_bf16_skinny");
@@ -227,6 +236,17 @@ static int skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int 
   return launch_skinny<4, 8, 1, 4, GATED>(a, w, c, out_dtype, M, N, K, st);
 }
 
+// Tile-major weights, M <= 16. Configurations from timing all of them on the shapes of the
+// 4B model: eight waves and eight steps in flight everywhere; two row tiles per block where
+// there are many tiles and no gate (the activations are then read half as often).
+template <bool GATED>
+static int skinny_tiled(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K,
+                        hipStream_t st) {
+  const int tiles = N / 16;
+  if (!GATED && tiles >= 384) return launch_skinny<1, 8, 2, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
+  return launch_skinny<1, 8, 1, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
+}
+
 template <int MT, int NT>
 static int launch(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K, hipStream_t stream) {
   dim3 grid((N + 64 * NT - 1) / (64 * NT), (M + 16 * MT - 1) / (16 * MT)), block(256);
@@ -241,16 +261,47 @@ static int launch(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int 
   return 0;
 }
 
+// Tuning aid: run one named configuration of the few-row kernel (M <= 16), so that
+// configurations can be timed against each other on the shapes of a model.
+extern "C" int qrt_gemm_bf16_variant(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K,
+                                     int gated, int variant, hipStream_t stream) {
+  QRT_CHECK(M >= 1 && M <= 16 && K % 32 == 0, "gemm_bf16_variant: M <= 16 and K a multiple of 32 only");
+  const bf16_t* A = (const bf16_t*)a;
+  const bf16_t* W = (const bf16_t*)w;
+#define V(ID, NW, NT, U)                                                                            \
+  if (variant == ID)                                                                                \
+    return gated ? launch_skinny<1, NW, NT, U, true>(A, W, c, out_dtype, M, N, K, stream)           \
+                 : launch_skinny<1, NW, NT, U, false>(A, W, c, out_dtype, M, N, K, stream);
+  V(0, 8, 1, 8) V(1, 8, 2, 8) V(2, 16, 1, 8) V(4, 4, 1, 8) V(10, 4, 1, 16)
+#undef V
+  // 100 + id: the same on tile-major weights
+#define V(ID, NW, NT, U)                                                                            \
+  if (variant == 100 + ID)                                                                          \
+    return gated ? launch_skinny<1, NW, NT, U, true, true>(A, W, c, out_dtype, M, N, K, stream)     \
+                 : launch_skinny<1, NW, NT, U, false, true>(A, W, c, out_dtype, M, N, K, stream);
+  V(0, 8, 1, 8) V(1, 8, 2, 8) V(2, 16, 1, 8) V(4, 4, 1, 8) V(10, 4, 1, 16)
+#undef V
+  return qrt_fail("gemm_bf16_variant: no variant %d", variant);
+}
+
 // gated = 0: C[M, N] = A W^T with W [N, K].
 // gated = 1: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A Wg^T) * (A Wu^T).
+// tiled = 1: W is stored tile-major, [rows / 16][K / 32][64 lanes][8]: lane q * 16 + i of tile
+// (r, s) holds W[16 r + i][32 s + 8 q .. + 7]; needs M <= 16, N % 16 == 0, K % 32 == 0.
 extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K, int gated,
-                             hipStream_t stream) {
+                             int tiled, hipStream_t stream) {
   QRT_CHECK(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   QRT_CHECK(gated == 0 || gated == 1, "gemm_bf16: unknown mode %d", gated);
   if (M == 0) return 0;
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
   const bool aligned = (K % 32 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
+  if (tiled) {
+    QRT_CHECK(M <= 16 && N % 16 == 0 && aligned,
+              "gemm_bf16: tile-major weights need M <= 16, N %% 16 == 0, K %% 32 == 0 (M=%d N=%d K=%d)", M, N, K);
+    return gated ? skinny_tiled<true>(A, W, c, out_dtype, M, N, K, stream)
+                 : skinny_tiled<false>(A, W, c, out_dtype, M, N, K, stream);
+  }
   if (M <= 64 && aligned) return gated ? skinny<true>(A, W, c, out_dtype, M, N, K, stream)
                                        : skinny<false>(A, W, c, out_dtype, M, N, K, stream);
   QRT_CHECK(gated == 0, "gemm_bf16: the gated form needs M <= 64 and K a multiple of 32 (M=%d K=%d)", M, K);

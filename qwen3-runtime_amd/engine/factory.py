@@ -65,7 +65,9 @@ def load(model_dir: str | Path | None, engine: EngineConfig, *, source=None, raw
         if device.type != "cuda":
             raise RuntimeError("the engine runs on a GPU only; there is no CPU path")
         ops = HipOps()
-    loader = load_model(model, source, device, dtype, where=f" in {model_dir}" if model_dir else "")
+    prepare = getattr(ops, "prepare_weight", None) if engine.decode_weight_copy else None
+    loader = load_model(model, source, device, dtype, where=f" in {model_dir}" if model_dir else "",
+                        prepare=prepare)
     num_pages = engine.num_pages or pages_for_memory(model, engine, dtype, device)
     cache = CacheManager(
         model.plan.caches, page_size=engine.page_size, num_pages=num_pages,

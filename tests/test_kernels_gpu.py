@@ -130,6 +130,38 @@ def test_gemm_bf16_few_rows_at_model_sizes(ops, m, n, k, own_max_rows, monkeypat
     close(ops.linear(x, w), want, 3e-2, 3e-2)
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+@pytest.mark.parametrize("n,k,gated", [(6144, 2560, False), (2560, 4096, False), (608, 9728, False), (64, 64, False),
+                                       (9728, 2560, True), (48, 96, True), (151936, 256, False)])
+def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
+    """A prepared weight (tile-major copy) gives the products of the plain one: both agree with a
+    float64 product (the two may add partial sums in different orders)."""
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    plain, prepared = HipOps(), HipOps()
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * n if gated else n, k, dtype=torch.bfloat16, seed=2, scale=0.03)
+    prepared.prepare_weight(w)
+    assert prepared._tiled_copy(w) is not None and plain._tiled_copy(w) is None
+    if gated:
+        want = R.swiglu((x.double() @ w.double().T).to(torch.bfloat16).double())
+        close(prepared.gated_linear(x, w), want, 3e-2, 3e-2)
+        close(plain.gated_linear(x, w), want, 3e-2, 3e-2)
+    else:
+        want = x.double() @ w.double().T
+        close(prepared.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
+        close(plain.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
+        close(prepared.linear(x, w), want, 3e-2, 3e-2)
+    # more rows than the few-row kernel takes: the copy is not used, the result is the library's
+    big = rnd(40, k, dtype=torch.bfloat16, seed=3)
+    if not gated:
+        assert torch.equal(prepared.linear(big, w), plain.linear(big, w))
+    # sizes that cannot be tiled are left alone
+    odd = rnd(24, 48, dtype=torch.bfloat16)
+    prepared.prepare_weight(odd)
+    assert prepared._tiled_copy(odd) is None
+
+
 def test_gemm_bf16_large_uses_blas_and_agrees(ops):
     x, w = rnd(300, 512, dtype=torch.bfloat16, seed=1), rnd(640, 512, dtype=torch.bfloat16, seed=2, scale=0.05)
     close(ops.linear(x, w), x.double() @ w.double().T, 3e-2, 3e-2)
