@@ -35,43 +35,123 @@ extern "C" int qrt_embed(const int* ids, const void* table, int table_dtype, flo
 // r = rows ? rows[b] : b
 // x = residual[r] (+ delta[r]);  without `rows` the sum is written back.
 // out[b] = x * rsqrt(mean(x^2) + eps) * weight
-template <typename TD, typename TO>
-__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
-                                   const float* __restrict__ weight, const int* __restrict__ rows,
-                                   TO* __restrict__ out, int hidden, float eps) {
-  extern __shared__ float xs[];  // hidden floats + 32 for the reduction
-  float* red = xs + hidden;
+// One block of 256 threads per row. Each thread keeps its elements of the row in registers
+// (rows up to 256 * VEC * KEEP wide; wider rows are read a second time), all loads of a row are
+// issued before the first use, squares are summed over the block in a fixed order.
+// delta may come as `planes` planes [planes, T, H] that are added in order (the parts of a product
+// whose K was cut).
+template <typename TD, typename TO, int VEC, int KEEP>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                                          const float* __restrict__ weight,
+                                                          const int* __restrict__ rows, TO* __restrict__ out,
+                                                          int hidden, float eps, int planes, size_t plane_stride) {
+  typedef float fvec_t __attribute__((ext_vector_type(VEC)));
+  typedef TD dvec_t __attribute__((ext_vector_type(VEC)));
+  typedef TO ovec_t __attribute__((ext_vector_type(VEC)));
+  __shared__ float red[32];
   const int b = blockIdx.x;
   const int r = rows ? rows[b] : b;
   float* res = residual + (size_t)r * hidden;
   const TD* del = delta ? delta + (size_t)r * hidden : nullptr;
+  const bool write_back = del && !rows;
+  constexpr int STRIDE = 256 * VEC;
+  const int i0 = threadIdx.x * VEC;
+
+  fvec_t x[KEEP];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    float x = res[i];
-    if (del) {
-      x += to_f32<TD>(del[i]);
-      if (!rows) res[i] = x;
-    }
-    xs[i] = x;
-    ss += x * x;
+#pragma unroll
+  for (int j = 0; j < KEEP; ++j) {
+    const int i = i0 + j * STRIDE;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) x[j][e] = 0.f;
+    if (i < hidden) x[j] = *(const fvec_t*)(res + i);
   }
-  const float total = block_sum(ss, red);
-  const float inv = rsqrtf(total / (float)hidden + eps);
+  if (del) {
+    for (int p = 0; p < planes; ++p) {
+#pragma unroll
+      for (int j = 0; j < KEEP; ++j) {
+        const int i = i0 + j * STRIDE;
+        if (i < hidden) {
+          const dvec_t d = *(const dvec_t*)(del + p * plane_stride + i);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) x[j][e] += to_f32<TD>(d[e]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < KEEP; ++j) {
+    const int i = i0 + j * STRIDE;
+    if (i < hidden) {
+      if (write_back) *(fvec_t*)(res + i) = x[j];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) ss += x[j][e] * x[j][e];
+    }
+  }
+  // the part of a row beyond what the registers hold
+  for (int i = i0 + KEEP * STRIDE; i < hidden; i += STRIDE) {
+    fvec_t v = *(const fvec_t*)(res + i);
+    if (del) {
+      for (int p = 0; p < planes; ++p) {
+        const dvec_t d = *(const dvec_t*)(del + p * plane_stride + i);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] += to_f32<TD>(d[e]);
+      }
+      if (write_back) *(fvec_t*)(res + i) = v;
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) ss += v[e] * v[e];
+  }
+  const float inv = rsqrtf(block_sum(ss, red) / (float)hidden + eps);
   TO* o = out + (size_t)b * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_f32<TO>(xs[i] * inv * weight[i]);
+#pragma unroll
+  for (int j = 0; j < KEEP; ++j) {
+    const int i = i0 + j * STRIDE;
+    if (i < hidden) {
+      const fvec_t w = *(const fvec_t*)(weight + i);
+      ovec_t y;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) y[e] = from_f32<TO>(x[j][e] * inv * w[e]);
+      *(ovec_t*)(o + i) = y;
+    }
+  }
+  for (int i = i0 + KEEP * STRIDE; i < hidden; i += STRIDE) {
+    fvec_t v = *(const fvec_t*)(res + i);  // already summed if written back
+    if (del && !write_back) {
+      for (int p = 0; p < planes; ++p) {
+        const dvec_t d = *(const dvec_t*)(del + p * plane_stride + i);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] += to_f32<TD>(d[e]);
+      }
+    }
+    const fvec_t w = *(const fvec_t*)(weight + i);
+    ovec_t y;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) y[e] = from_f32<TO>(v[e] * inv * w[e]);
+    *(ovec_t*)(o + i) = y;
+  }
 }
 
 extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dtype, const float* weight,
                                const int* rows, void* out, int out_dtype, int num_out_rows, int hidden,
-                               float eps, hipStream_t stream) {
+                               float eps, int planes, long plane_stride, hipStream_t stream) {
   QRT_CHECK(hidden > 0 && num_out_rows >= 0, "add_rmsnorm: bad sizes rows=%d H=%d", num_out_rows, hidden);
-  const size_t smem = ((size_t)hidden + 32) * sizeof(float);
-  QRT_CHECK(smem <= 64 * 1024, "add_rmsnorm: width %d needs %zu bytes of LDS, limit 65536", hidden, smem);
+  QRT_CHECK(planes >= 1 && planes <= 64 && plane_stride >= 0, "add_rmsnorm: bad delta planes %d", planes);
   if (num_out_rows == 0) return 0;
-  dim3 grid(num_out_rows), block(hidden >= 2048 ? 512 : 256);
-#define LAUNCH(TD, TO)                                                                    \
-  add_rmsnorm_kernel<TD, TO><<<grid, block, smem, stream>>>(residual, (const TD*)delta, weight, rows, \
-                                                            (TO*)out, hidden, eps)
+  dim3 grid(num_out_rows), block(256);
+  const bool vec4 = hidden % 4 == 0 && (uintptr_t)residual % 16 == 0 && (uintptr_t)weight % 16 == 0 &&
+                    (uintptr_t)out % 16 == 0 && (!delta || (uintptr_t)delta % 16 == 0) && plane_stride % 4 == 0;
+#define LAUNCH(TD, TO)                                                                                          \
+  do {                                                                                                          \
+    if (vec4)                                                                                                   \
+      add_rmsnorm_kernel<TD, TO, 4, 4><<<grid, block, 0, stream>>>(residual, (const TD*)delta, weight, rows,    \
+                                                                   (TO*)out, hidden, eps, planes,               \
+                                                                   (size_t)plane_stride);                       \
+    else                                                                                                        \
+      add_rmsnorm_kernel<TD, TO, 1, 8><<<grid, block, 0, stream>>>(residual, (const TD*)delta, weight, rows,    \
+                                                                   (TO*)out, hidden, eps, planes,               \
+                                                                   (size_t)plane_stride);                       \
+  } while (0)
   if (delta_dtype == QRT_F32 && out_dtype == QRT_F32) LAUNCH(float, float);
   else if (delta_dtype == QRT_BF16 && out_dtype == QRT_BF16) LAUNCH(bf16_t, bf16_t);
   else if (delta_dtype == QRT_F32 && out_dtype == QRT_BF16) LAUNCH(float, bf16_t);

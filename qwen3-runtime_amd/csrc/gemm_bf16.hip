@@ -140,11 +140,16 @@ __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t*
 #pragma unroll
     for (int b = 0; b < MB; ++b) acc[t][b] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  const int steps = K >> 5;  // K is a multiple of 32 here
+  // gridDim.y blocks share the row tiles; block y takes the y-th part of the k-steps and writes
+  // output plane y (the caller adds the planes: used where the result feeds a residual add)
+  const int all_steps = K >> 5;  // K is a multiple of 32 here
+  const int part = (all_steps + gridDim.y - 1) / gridDim.y;
+  const int s_first = blockIdx.y * part, steps = min(all_steps, s_first + part);
+  C += (size_t)blockIdx.y * M * N;
   bf16x8_t zero;
 #pragma unroll
   for (int e = 0; e < 8; ++e) zero[e] = (bf16_t)0.0f;
-  for (int s0 = wave; s0 < steps; s0 += U * NW) {
+  for (int s0 = s_first + wave; s0 < steps; s0 += U * NW) {
     bf16x8_t w[U][WT], a[U][MB];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -207,8 +212,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t*
 
 template <int MB, int NW, int NT, int U, bool GATED, bool TILED = false>
 static int launch_skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K,
-                         hipStream_t stream) {
-  dim3 grid((N + 16 * NT - 1) / (16 * NT)), block(64 * NW);
+                         hipStream_t stream, int k_parts = 1) {
+  dim3 grid((N + 16 * NT - 1) / (16 * NT), k_parts), block(64 * NW);
   const size_t smem = (size_t)NW * (GATED ? 2 : 1) * NT * MB * 4 * 64 * sizeof(float);
   if (out_dtype == QRT_BF16)
     gemm_bf16_skinny_kernel<MB, NW, NT, U, GATED, TILED, bf16_t><<<grid, block, smem, stream>>>(a, w, (bf16_t*)c, M, N, K);
@@ -241,10 +246,11 @@ static int skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int 
 // there are many tiles and no gate (the activations are then read half as often).
 template <bool GATED>
 static int skinny_tiled(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K,
-                        hipStream_t st) {
+                        hipStream_t st, int k_parts) {
   const int tiles = N / 16;
-  if (!GATED && tiles >= 384) return launch_skinny<1, 8, 2, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
-  return launch_skinny<1, 8, 1, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
+  if (!GATED && tiles >= 384 && k_parts == 1)
+    return launch_skinny<1, 8, 2, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
+  return launch_skinny<1, 8, 1, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st, k_parts);
 }
 
 template <int MT, int NT>
@@ -288,10 +294,15 @@ extern "C" int qrt_gemm_bf16_variant(const void* a, const void* w, void* c, int 
 // gated = 1: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A Wg^T) * (A Wu^T).
 // tiled = 1: W is stored tile-major, [rows / 16][K / 32][64 lanes][8]: lane q * 16 + i of tile
 // (r, s) holds W[16 r + i][32 s + 8 q .. + 7]; needs M <= 16, N % 16 == 0, K % 32 == 0.
+// k_parts > 1 (tile-major, not gated, float32 out): K is cut into that many parts, each handled
+// by blocks of its own, and C is [k_parts, M, N]: planes to be added by the caller.
 extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K, int gated,
-                             int tiled, hipStream_t stream) {
+                             int tiled, int k_parts, hipStream_t stream) {
   QRT_CHECK(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   QRT_CHECK(gated == 0 || gated == 1, "gemm_bf16: unknown mode %d", gated);
+  QRT_CHECK(k_parts >= 1 && k_parts <= 64, "gemm_bf16: bad number of K parts %d", k_parts);
+  QRT_CHECK(k_parts == 1 || (tiled && !gated && out_dtype == QRT_F32),
+            "gemm_bf16: K parts need tile-major weights, no gate and float32 output");
   if (M == 0) return 0;
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
@@ -299,8 +310,8 @@ extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtyp
   if (tiled) {
     QRT_CHECK(M <= 16 && N % 16 == 0 && aligned,
               "gemm_bf16: tile-major weights need M <= 16, N %% 16 == 0, K %% 32 == 0 (M=%d N=%d K=%d)", M, N, K);
-    return gated ? skinny_tiled<true>(A, W, c, out_dtype, M, N, K, stream)
-                 : skinny_tiled<false>(A, W, c, out_dtype, M, N, K, stream);
+    return gated ? skinny_tiled<true>(A, W, c, out_dtype, M, N, K, stream, 1)
+                 : skinny_tiled<false>(A, W, c, out_dtype, M, N, K, stream, k_parts);
   }
   if (M <= 64 && aligned) return gated ? skinny<true>(A, W, c, out_dtype, M, N, K, stream)
                                        : skinny<false>(A, W, c, out_dtype, M, N, K, stream);

@@ -178,8 +178,13 @@ class HipOps:
         t, h = residual.shape
         _need(residual, "residual", torch.float32)
         _need(weight, "norm weight", torch.float32, (h,))
+        planes, plane_stride = 1, 0
         if delta is not None:
-            _need(delta, "delta", shape=(t, h))
+            if delta.dim() == 3:  # the parts of a product whose K was cut: added here, in order
+                planes, plane_stride = delta.shape[0], t * h
+                _need(delta, "delta", shape=(planes, t, h))
+            else:
+                _need(delta, "delta", shape=(t, h))
         n_out = t
         if rows is not None:
             _need(rows, "rows", torch.int32)
@@ -187,7 +192,8 @@ class HipOps:
         out = torch.empty((n_out, h), dtype=out_dtype, device=residual.device)
         self._check(self.lib, self.lib.qrt_add_rmsnorm(
             _ptr(residual), _ptr(delta), _CODE[delta.dtype] if delta is not None else F32, _ptr(weight),
-            _ptr(rows), _ptr(out), _CODE[out_dtype], c_int(n_out), c_int(h), c_float(eps), _stream()))
+            _ptr(rows), _ptr(out), _CODE[out_dtype], c_int(n_out), c_int(h), c_float(eps), c_int(planes),
+            c_long(plane_stride), _stream()))
         return out
 
     def swiglu(self, gate_up):
@@ -227,8 +233,35 @@ class HipOps:
         tiled = self._tiled_copy(w)
         self._check(self.lib, self.lib.qrt_gemm_bf16(
             _ptr(x), _ptr(w if tiled is None else tiled), _ptr(out), F32 if out_f32 else BF16,
-            c_int(m), c_int(n), c_int(k), c_int(0), c_int(0 if tiled is None else 1), _stream()))
+            c_int(m), c_int(n), c_int(k), c_int(0), c_int(0 if tiled is None else 1), c_int(1), _stream()))
         return out
+
+    def linear_for_residual(self, x, w):
+        """``linear(x, w)`` for a result that is only ever added to the residual stream.
+
+        May return the result in planes ``[P, T, N]`` float32 whose sum it is (``add_rmsnorm``
+        adds them): a product with few rows and few weight rows then cuts K over several blocks
+        per row tile, which fills the chip (160 row tiles for 256 compute units at the 4B size)."""
+        m, k = x.shape
+        n = w.shape[0]
+        tiled = self._tiled_copy(w) if (x.dtype == torch.bfloat16 and m <= self.own_max_rows) else None
+        parts = self.choose_k_parts(n, k) if tiled is not None else 1
+        if parts == 1:
+            return self.linear(x, w)
+        _need(x, "x", torch.bfloat16)
+        out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+        self._check(self.lib, self.lib.qrt_gemm_bf16(
+            _ptr(x), _ptr(tiled), _ptr(out), F32, c_int(m), c_int(n), c_int(k), c_int(0), c_int(1),
+            c_int(parts), _stream()))
+        return out
+
+    @staticmethod
+    def choose_k_parts(n: int, k: int) -> int:
+        """Cut K when there are fewer row tiles than about two per compute unit and K is long."""
+        tiles = n // 16
+        if tiles >= 384 or k < 2048:
+            return 1
+        return 2 if k < 8192 else 4
 
     # rows up to which the gated activation is fused into the product before it
     fused_gate_max_rows = 16
@@ -249,7 +282,7 @@ class HipOps:
             tiled = self._tiled_copy(w_gate_up) if (two_i // 2) % 16 == 0 else None
             self._check(self.lib, self.lib.qrt_gemm_bf16(
                 _ptr(x), _ptr(w_gate_up if tiled is None else tiled), _ptr(out), BF16, c_int(m),
-                c_int(two_i // 2), c_int(k), c_int(1), c_int(0 if tiled is None else 1), _stream()))
+                c_int(two_i // 2), c_int(k), c_int(1), c_int(0 if tiled is None else 1), c_int(1), _stream()))
             return out
         return self.swiglu(self.linear(x, w_gate_up))
 

@@ -98,4 +98,4 @@ class GroupedQueryAttention(Mixer):
                 ops.kv_store(k, v, cache)
             q = q.reshape(ctx.num_tokens, nq * d)
         attn = ops.paged_attention(q, cache, ctx, nq, nkv, d, self.scale, self.window)
-        return ops.linear(attn, self.o)
+        return ops.linear_for_residual(attn, self.o)

@@ -18,7 +18,8 @@ Roles and the call each must answer (``T`` tokens of this step, ``H`` width):
 
 The residual stream is float32 in every mode; ``delta`` is the output of the
 previous sub-layer that has not been added yet, so that the add fuses with the
-next norm.
+next norm. A sub-layer may hand its output over in planes ``[P, T, H]`` whose
+sum it is (``ops.linear_for_residual``); only a norm ever looks into ``delta``.
 """
 
 from __future__ import annotations

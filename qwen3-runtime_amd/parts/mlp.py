@@ -36,4 +36,4 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx, x):
         act = ctx.ops.gated_linear(x, self.gate_up)
-        return ctx.ops.linear(act, self.down)
+        return ctx.ops.linear_for_residual(act, self.down)

@@ -22,6 +22,8 @@ def embed(ids, table):
 
 
 def add_rmsnorm(residual, delta, weight, eps, out_dtype, rows=None, compute=torch.float32):
+    if delta is not None and delta.dim() == 3:
+        delta = delta.to(residual.dtype).sum(0)
     if delta is not None:
         if rows is None:
             residual += delta.to(residual.dtype)
@@ -159,6 +161,9 @@ class TorchOps:
 
     def linear(self, x, w, out_f32=False):
         return linear(x, w, out_f32, self.compute)
+
+    def linear_for_residual(self, x, w):
+        return linear(x, w, False, self.compute)
 
     def qk_norm_rope_store(self, qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions, cache):
         if cache is None:

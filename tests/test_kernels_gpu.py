@@ -162,6 +162,39 @@ def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
     assert prepared._tiled_copy(odd) is None
 
 
+@pytest.mark.parametrize("m", [1, 8, 16, 40])
+@pytest.mark.parametrize("n,k", [(2560, 4096), (2560, 9728), (96, 2048), (6144, 2560), (64, 64)])
+def test_product_for_the_residual_may_come_in_planes(m, n, k):
+    """linear_for_residual's planes sum to the product, and add_rmsnorm adds them like one delta."""
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    ops = HipOps()
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    w = rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.03)
+    ops.prepare_weight(w)
+    want = x.double() @ w.double().T
+    got = ops.linear_for_residual(x, w)
+    if m <= 16 and n // 16 < 384 and k >= 2048:
+        assert got.dim() == 3 and got.shape[0] == ops.choose_k_parts(n, k) > 1 and got.dtype == torch.float32
+        close(got.sum(0), want, 2e-3, 2e-3)
+    else:
+        assert got.dim() == 2
+        close(got, want, 3e-2, 3e-2)
+    res = rnd(m, n, seed=4)
+    weight = (1 + 0.1 * rnd(n, seed=5)).contiguous()
+    one = got if got.dim() == 2 else got.sum(0).to(torch.bfloat16)
+    res_a, res_b = res.clone(), res.clone()
+    ya = ops.add_rmsnorm(res_a, got, weight, 1e-6, torch.bfloat16)
+    yb = ops.add_rmsnorm(res_b, one, weight, 1e-6, torch.bfloat16)
+    close(res_a, res_b, 2e-2, 2e-2)
+    close(ya, yb, 3e-2, 3e-2)
+    want_res = res.double() + want
+    close(res_a, want_res, 3e-2, 3e-2)
+    rows = torch.tensor([m - 1, 0], dtype=torch.int32, device=DEV)
+    yc = ops.add_rmsnorm(res.clone(), got, weight, 1e-6, torch.bfloat16, rows)
+    close(yc, ya[rows.long()], 0, 0)
+
+
 def test_gemm_bf16_large_uses_blas_and_agrees(ops):
     x, w = rnd(300, 512, dtype=torch.bfloat16, seed=1), rnd(640, 512, dtype=torch.bfloat16, seed=2, scale=0.05)
     close(ops.linear(x, w), x.double() @ w.double().T, 3e-2, 3e-2)
