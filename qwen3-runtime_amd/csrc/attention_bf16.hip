@@ -62,6 +62,7 @@ struct AttnTileArgs {
   int table_width, num_tiles, nq, nkv, page_size, window, num_splits, waves;
   float scale_log2;
   int row_tiles;  // tiles of 16 rows per wave (general kernel): 1, 2 or 4
+  int use_lds;    // long portions: share keys and values of a block of waves through LDS
 };
 
 constexpr int D = QRT_HEAD_DIM;
@@ -69,12 +70,77 @@ constexpr int KFULL = D / 32;        // 32-wide steps of the first product
 constexpr bool KTAIL = (D % 32) != 0;  // one 16-wide step more
 constexpr int DB = D / 16;           // 16-wide blocks of the head dimension
 
+// One tile of 16 rows meets one block of 32 keys: sc holds the raw scores (this lane: its row,
+// keys base + 8 quad + e), vv the block's values as MFMA operands. Online softmax in base 2;
+// the running maximum m is kept in scaled units (score * scale * log2 e). masked = false is for
+// blocks every row of the tile sees in full, the common case away from the diagonal: no compare,
+// no select. The rescale of the accumulator is skipped when no row's maximum moved.
+// The scale is positive (checked on the host), so the maximum may be taken before scaling.
+// Position -> (page of the block table, offset in the page). Division by a run-time number
+// costs some thirty instructions per use; page sizes are powers of two in practice, so the
+// kernels are built twice: P2 = true shifts and masks, P2 = false divides.
+template <bool P2> __device__ __forceinline__ int page_div(int x, int ps, int shift) { return P2 ? x >> shift : x / ps; }
+template <bool P2> __device__ __forceinline__ int page_mod(int x, int ps) { return P2 ? x & (ps - 1) : x % ps; }
+
+// max over the four lanes that hold one row (lane, lane ^ 16, lane ^ 32, lane ^ 48): two swaps of
+// register halves between rows of 16 lanes, no LDS traffic and no address arithmetic
+__device__ __forceinline__ float row_max4(float x) {
+  typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+  const unsigned int u = __float_as_uint(x);
+  const u32x2_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const unsigned int v = __float_as_uint(y);
+  const u32x2_t b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+__device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t* vv, bool masked, int base,
+                                            int quad, bool row_valid, int qpos, int window, float scale_log2,
+                                            float& m, float& l, f32x4_t* o) {
+  float s[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) s[e] = sc[e >> 2][e & 3];
+  if (masked) {  // the same for the whole wave
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = base + 8 * quad + e;
+      const bool vis = row_valid && key <= qpos && (window == 0 || key > qpos - window);
+      s[e] = vis ? s[e] : -INFINITY;
+    }
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) mx = fmaxf(mx, s[e]);
+  mx = row_max4(mx);
+  const float m_new = fmaxf(m, mx * scale_log2);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
+  // v_exp_f32 directly: results below the normal range may flush to zero, which is what they are worth here
+  const float corr = __builtin_amdgcn_exp2f(m - m_use);
+  float psum = 0.f;
+  bf16x8_t pb;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float pe = __builtin_amdgcn_exp2f(fmaf(s[e], scale_log2, -m_use));
+    psum += pe;
+    pb[e] = (bf16_t)pe;
+  }
+  m = m_new;
+  if (__any(corr != 1.0f)) {
+    l *= corr;
+#pragma unroll
+    for (int i = 0; i < DB; ++i) o[i] *= corr;
+  }
+  l += psum;
+#pragma unroll
+  for (int i = 0; i < DB; ++i) o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[i], pb, o[i], 0, 0, 0);
+}
+
 // General kernel (prompt portions and mixed batches). A wave owns RT tiles of 16
 // rows each, 16 * RT consecutive rows of the sequence's row matrix; a block is
 // four waves, 64 * RT rows. The keys and values of a block of 32 keys are read
 // once into registers and multiplied with all RT tiles, which divides the
 // operand traffic per MFMA by RT.
-template <int RT>
+template <int RT, bool P2>
 __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(AttnTileArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
@@ -88,12 +154,12 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
   const int row0 = a.tile_row0[blockIdx.x] + 16 * RT * wave;
   if (row0 >= n_rows) return;
   const int first_pos = kv_len - q_len;
-  const int ps = a.page_size;
+  const int ps = a.page_size, psh = __builtin_ctz(ps);
   const int* table = a.block_table + (size_t)seq * a.table_width;
 
   // per tile: this lane's row, its token's position, and Q as B operands kept for the whole loop
   bool row_valid[RT];
-  int qpos[RT];
+  int qpos[RT], tile_pos_min[RT], tile_pos_max[RT];  // this lane's position; the tile's range of positions
   size_t row_index[RT];
   bf16x8_t qreg[RT][KFULL > 0 ? KFULL : 1];
   bf16x8_t qtail[RT];
@@ -104,6 +170,9 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
     const int row_c = row_valid[t] ? my_row : n_rows - 1;
     const int tok = row_c / g, hg = row_c - tok * g;
     qpos[t] = first_pos + tok;
+    // the same for every lane: kept in scalar registers so that the choice below is a plain branch
+    tile_pos_min[t] = __builtin_amdgcn_readfirstlane(first_pos + min(row0 + 16 * t, n_rows - 1) / g);
+    tile_pos_max[t] = __builtin_amdgcn_readfirstlane(first_pos + min(row0 + 16 * t + 15, n_rows - 1) / g);
     row_index[t] = (size_t)(q_begin + tok) * a.nq + kvh * g + hg;
     const bf16_t* qp = a.q + row_index[t] * D;
 #pragma unroll
@@ -139,8 +208,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
     for (int kb = 0; kb < 2; ++kb) {
       int kidx = base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3);
       kidx = min(max(kidx, lo), pos_max);  // stay inside pages this sequence holds; masked below
-      const int page = table[kidx / ps];
-      const bf16_t* kp = a.k_cache + (((size_t)page * a.nkv + kvh) * ps + (kidx % ps)) * D;
+      const int page = table[page_div<P2>(kidx, ps, psh)];
+      const bf16_t* kp = a.k_cache + (((size_t)page * a.nkv + kvh) * ps + page_mod<P2>(kidx, ps)) * D;
 #pragma unroll
       for (int i = 0; i < KFULL; ++i) kk[kb][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
       if (KTAIL) kt[kb] = load_tail(kp + 32 * KFULL, quad);
@@ -148,8 +217,8 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
     // values: 8 consecutive keys base + 8 quad .. + 7 of head element 16 i + r16
     const int kv0 = base + 8 * quad;
     const bool vload = kv0 <= pos_max && kv0 + 7 >= lo;
-    const int vpage = vload ? table[kv0 / ps] : 0;
-    const bf16_t* vp = a.v_cache + (((size_t)vpage * a.nkv + kvh) * D + r16) * ps + (kv0 % ps);
+    const int vpage = vload ? table[page_div<P2>(kv0, ps, psh)] : 0;
+    const bf16_t* vp = a.v_cache + (((size_t)vpage * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps);
     bf16x8_t vv[DB];
 #pragma unroll
     for (int i = 0; i < DB; ++i) {
@@ -172,36 +241,9 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
         if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[kb], qtail[t], acc, 0, 0, 0);
         s[kb] = acc;
       }
-      // this lane: row r16 of tile t, keys base + 8 quad + 4 kb + r
-      float p[8];
-      float mx = -INFINITY;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int key = base + 8 * quad + e;
-        const bool vis = row_valid[t] && key <= qpos[t] && (a.window == 0 || key > qpos[t] - a.window);
-        p[e] = vis ? s[e >> 2][e & 3] * a.scale_log2 : -INFINITY;
-        mx = fmaxf(mx, p[e]);
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[t], mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float corr = exp2f(m[t] - m_use);
-      float psum = 0.f;
-      bf16x8_t pb;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float pe = exp2f(p[e] - m_use);
-        psum += pe;
-        pb[e] = (bf16_t)pe;
-      }
-      l[t] = l[t] * corr + psum;
-      m[t] = m_new;
-#pragma unroll
-      for (int i = 0; i < DB; ++i) {
-        o[t][i] *= corr;
-        o[t][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[i], pb, o[t][i], 0, 0, 0);
-      }
+      // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
+      const bool whole = base + 31 <= tile_pos_min[t] && (a.window == 0 || base > tile_pos_max[t] - a.window);
+      tile_update(s, vv, !whole, base, quad, row_valid[t], qpos[t], a.window, a.scale_log2, m[t], l[t], o[t]);
     }
   }
 
@@ -229,6 +271,213 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
         *(f32x4_t*)(op + 16 * i + 4 * quad) = w;
       }
       if (quad == 0) a.part_lse[row_index[t] * a.num_splits + split] = lt > 0.f ? m[t] + log2f(lt) : -INFINITY;
+    }
+  }
+}
+
+// Long portions: the same tiling (a wave owns RT tiles of 16 rows, a block four waves), but the
+// keys and values of a block of 32 keys are brought into LDS once per block of waves instead
+// of once per wave, and the next block's loads are in flight while the current one is
+// multiplied: 256 threads each fetch a few 16-byte pieces into registers, the waves multiply
+// from the other LDS stage, then the registers are stored and one barrier ends the round.
+// LDS rows are padded (keys: D + 8 elements, transposed values: 32 + 8 keys) so that the 16
+// lanes that read one MFMA operand together hit 16 different groups of banks.
+constexpr int KROW = D + 8;                // elements per key row in LDS
+constexpr int VROW = 40;                   // elements per value row (one head element, 32 keys) in LDS
+constexpr int PIECES = (4 * D + 255) / 256;  // 16-byte pieces per thread per operand and block
+constexpr int STAGE_ELEMS = 32 * KROW + D * VROW;
+
+template <int RT, bool P2>
+__global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTileArgs a) {
+  extern __shared__ bf16_t lds_kv[];  // [2][STAGE_ELEMS]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int seq = a.tile_seq[blockIdx.x];
+  const int kvh = blockIdx.y;
+  const int g = a.nq / a.nkv;
+  const int q_begin = a.cu_q[seq];
+  const int q_len = a.cu_q[seq + 1] - q_begin;
+  const int kv_len = a.kv_lens[seq];
+  const int n_rows = q_len * g;
+  const int tile_row0 = a.tile_row0[blockIdx.x];  // first row of the block of waves; < n_rows
+  const int row0 = tile_row0 + 16 * RT * wave;
+  const bool wave_has_rows = row0 < n_rows;
+  const int first_pos = kv_len - q_len;
+  const int ps = a.page_size, psh = __builtin_ctz(ps);
+  const int* table = a.block_table + (size_t)seq * a.table_width;
+
+  bool row_valid[RT];
+  int qpos[RT], tile_pos_min[RT], tile_pos_max[RT];  // this lane's position; the tile's range of positions
+  size_t row_index[RT];
+  bf16x8_t qreg[RT][KFULL > 0 ? KFULL : 1];
+  bf16x8_t qtail[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    const int my_row = row0 + 16 * t + r16;
+    row_valid[t] = my_row < n_rows;
+    const int row_c = min(my_row, n_rows - 1);
+    const int tok = row_c / g, hg = row_c - tok * g;
+    qpos[t] = first_pos + tok;
+    // the same for every lane: kept in scalar registers so that the choice below is a plain branch
+    tile_pos_min[t] = __builtin_amdgcn_readfirstlane(first_pos + min(row0 + 16 * t, n_rows - 1) / g);
+    tile_pos_max[t] = __builtin_amdgcn_readfirstlane(first_pos + min(row0 + 16 * t + 15, n_rows - 1) / g);
+    row_index[t] = (size_t)(q_begin + tok) * a.nq + kvh * g + hg;
+    const bf16_t* qp = a.q + row_index[t] * D;
+#pragma unroll
+    for (int i = 0; i < KFULL; ++i) qreg[t][i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
+    qtail[t] = load_tail(qp, 2);  // zeros
+    if (KTAIL) qtail[t] = load_tail(qp + 32 * KFULL, quad);
+  }
+
+  // keys the block of waves needs, and the part of them this wave needs
+  const int blk_last_row = min(tile_row0 + 64 * RT - 1, n_rows - 1);
+  const int blk_pos_min = first_pos + tile_row0 / g, blk_pos_max = first_pos + blk_last_row / g;
+  const int lo = a.window > 0 ? max(0, blk_pos_min - a.window + 1) : 0;
+  const int b0 = lo >> 5, b1 = (blk_pos_max >> 5) + 1;
+  int wb0 = b1, wb1 = b0;  // this wave's blocks: none unless it has rows
+  if (wave_has_rows) {
+    const int row_last = min(row0 + 16 * RT - 1, n_rows - 1);
+    const int pos_min = first_pos + row0 / g, pos_max = first_pos + row_last / g;
+    wb0 = (a.window > 0 ? max(0, pos_min - a.window + 1) : 0) >> 5;
+    wb1 = (pos_max >> 5) + 1;
+  }
+
+  f32x4_t o[RT][DB];
+  float m[RT], l[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    m[t] = -INFINITY;
+    l[t] = 0.f;
+#pragma unroll
+    for (int i = 0; i < DB; ++i) o[t][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  }
+
+  // Block table entries are looked up one round before the loads that need them, so that no
+  // load waits for another: lookup(b + 2) and fetch(b + 1) are in flight while block b is multiplied.
+  const size_t page_stride = (size_t)a.nkv * ps * D;  // elements per page, keys and values alike
+  const bf16_t* k_head = a.k_cache + (size_t)kvh * ps * D;
+  const bf16_t* v_head = a.v_cache + (size_t)kvh * D * ps;
+  bf16x8_t kpiece[PIECES], vpiece[PIECES];
+  // Every load below is unconditional (indices are clamped into pages the sequence holds, what
+  // lies outside is zeroed by a select): with loads under branches the compiler can no longer
+  // count which are in flight and waits for all of them in the middle of the products.
+  constexpr bool ALL_THREADS = (4 * D) % 256 == 0;  // every thread has PIECES pieces
+  auto lookup = [&](int b, int* kpage, int* vpage) {
+    const int base = b << 5;
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (ALL_THREADS || c < 4 * D) {
+        const int kidx = min(max(base + c / (D / 8), lo), blk_pos_max);  // masked later where clamped
+        kpage[i] = table[page_div<P2>(kidx, ps, psh)];
+        const int kv0 = min(max(base + 8 * (c & 3), lo & ~7), blk_pos_max & ~7);
+        vpage[i] = table[page_div<P2>(kv0, ps, psh)];
+      }
+    }
+  };
+  auto fetch = [&](int b, const int* kpage, const int* vpage) {  // global -> registers: this thread's pieces of block b
+    const int base = b << 5;
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (ALL_THREADS || c < 4 * D) {
+        const int key = c / (D / 8), part = c - key * (D / 8);
+        const int kidx = min(max(base + key, lo), blk_pos_max);
+        kpiece[i] = *(const bf16x8_t*)(k_head + (size_t)kpage[i] * page_stride + (page_mod<P2>(kidx, ps) * D + 8 * part));
+        const int d = c >> 2, kv0 = min(max(base + 8 * (c & 3), lo & ~7), blk_pos_max & ~7);
+        vpiece[i] = *(const bf16x8_t*)(v_head + (size_t)vpage[i] * page_stride + (d * ps + page_mod<P2>(kv0, ps)));
+      }
+    }
+  };
+  auto stash = [&](int b, int stage) {  // registers -> LDS: block b into its stage
+    bf16_t* kb = lds_kv + stage * STAGE_ELEMS;
+    bf16_t* vb = kb + 32 * KROW;
+    const int base = b << 5;
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (ALL_THREADS || c < 4 * D) {
+        const int key = c / (D / 8), part = c - key * (D / 8);
+        // row 16 s2 + r16 of the stage holds the key that lane r16 of sub-block s2 multiplies:
+        // the 16 lanes of an operand read 16 consecutive padded rows, all in different banks
+        const int row = 16 * ((key >> 2) & 1) + 4 * (key >> 3) + (key & 3);
+        *(bf16x8_t*)(kb + row * KROW + 8 * part) = kpiece[i];
+        const int d = c >> 2, j = c & 3;
+        // values of keys no row of the block sees were read from a clamped place: they may be
+        // anything, and 0 * NaN is NaN, so they become zeros
+        const int kv0 = base + 8 * j;
+        const bool seen = kv0 <= blk_pos_max && kv0 + 7 >= lo;
+        bf16x8_t v = vpiece[i];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = seen ? v[e] : (bf16_t)0.0f;
+        *(bf16x8_t*)(vb + d * VROW + 8 * j) = v;
+      }
+    }
+  };
+
+  int kpage[PIECES], vpage[PIECES];
+  lookup(b0, kpage, vpage);
+  fetch(b0, kpage, vpage);
+  if (b0 + 1 < b1) lookup(b0 + 1, kpage, vpage);
+  stash(b0, 0);
+  __syncthreads();
+  for (int b = b0; b < b1; ++b) {
+    const int stage = (b - b0) & 1;
+    if (b + 1 < b1) fetch(b + 1, kpage, vpage);      // with the entries the last round looked up
+    if (b + 2 < b1) lookup(b + 2, kpage, vpage);     // in flight until the next round
+    if (b >= wb0 && b < wb1) {  // uniform over the wave
+      const int base = b << 5;
+      const bf16_t* kb = lds_kv + stage * STAGE_ELEMS;
+      const bf16_t* vb = kb + 32 * KROW;
+      bf16x8_t kk[2][KFULL > 0 ? KFULL : 1], kt[2];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const bf16_t* kp = kb + (16 * s2 + r16) * KROW;
+#pragma unroll
+        for (int i = 0; i < KFULL; ++i) kk[s2][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
+        if (KTAIL) {
+          kt[s2] = load_tail(kp, 2);
+          if (quad < 2) kt[s2] = *(const bf16x8_t*)(kp + 32 * KFULL + 8 * quad);
+        }
+      }
+      bf16x8_t vv[DB];
+#pragma unroll
+      for (int i = 0; i < DB; ++i) vv[i] = *(const bf16x8_t*)(vb + (16 * i + r16) * VROW + 8 * quad);
+
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        f32x4_t sc[2];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < KFULL; ++i)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk[s2][i], qreg[t][i], acc, 0, 0, 0);
+          if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[s2], qtail[t], acc, 0, 0, 0);
+          sc[s2] = acc;
+        }
+        const bool whole = base + 31 <= tile_pos_min[t] && (a.window == 0 || base > tile_pos_max[t] - a.window);
+        tile_update(sc, vv, !whole, base, quad, row_valid[t], qpos[t], a.window, a.scale_log2, m[t], l[t], o[t]);
+      }
+    }
+    if (b + 1 < b1) stash(b + 1, stage ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    float lt = l[t];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    if (!row_valid[t]) continue;
+    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    bf16_t* op = a.out + row_index[t] * D;
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+      bf16x4_t w;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) w[r] = (bf16_t)(o[t][i][r] * inv);
+      *(bf16x4_t*)(op + 16 * i + 4 * quad) = w;
     }
   }
 }
@@ -273,36 +522,40 @@ struct KvBlock {  // the keys of one block, as MFMA operands
   bf16x8_t kt[2];
 };
 
+template <bool P2>
 __device__ __forceinline__ void block_pages(const int* __restrict__ table, int base, int lo, int pos_max, int ps,
                                             int r16, int quad, int pg[3]) {
+  const int psh = __builtin_ctz(ps);
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
     const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
-    pg[kb] = table[kidx / ps];
+    pg[kb] = table[page_div<P2>(kidx, ps, psh)];
   }
   const int kv0 = base + 8 * quad;
-  pg[2] = (kv0 <= pos_max && kv0 + 7 >= lo) ? table[kv0 / ps] : -1;
+  pg[2] = (kv0 <= pos_max && kv0 + 7 >= lo) ? table[page_div<P2>(kv0, ps, psh)] : -1;
 }
 
+template <bool P2>
 __device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int base, int lo, int pos_max, int r16,
                                            int quad, const int pg[3], KvBlock& blk) {
-  const int ps = a.page_size;
+  const int ps = a.page_size, psh = __builtin_ctz(ps);
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
     const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
-    const bf16_t* kp = a.k_cache + (((size_t)pg[kb] * a.nkv + kvh) * ps + (kidx % ps)) * D;
+    const bf16_t* kp = a.k_cache + (((size_t)pg[kb] * a.nkv + kvh) * ps + page_mod<P2>(kidx, ps)) * D;
 #pragma unroll
     for (int i = 0; i < KFULL; ++i) blk.k[kb][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
     if (KTAIL) blk.kt[kb] = load_tail(kp + 32 * KFULL, quad);
   }
 }
 
+template <bool P2>
 __device__ __forceinline__ void block_load_values(const AttnTileArgs& a, int kvh, int base, int r16, int quad,
                                                   int vpage, bf16x8_t* v) {
-  const int ps = a.page_size;
+  const int ps = a.page_size, psh = __builtin_ctz(ps);
   const int kv0 = base + 8 * quad;
   const bool vload = vpage >= 0;
-  const bf16_t* vp = a.v_cache + (((size_t)(vload ? vpage : 0) * a.nkv + kvh) * D + r16) * ps + (kv0 % ps);
+  const bf16_t* vp = a.v_cache + (((size_t)(vload ? vpage : 0) * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps);
 #pragma unroll
   for (int i = 0; i < DB; ++i) {
     if (vload) v[i] = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
@@ -356,6 +609,7 @@ __device__ __forceinline__ void block_compute(const KvBlock& blk, const bf16x8_t
   }
 }
 
+template <bool P2>
 __global__ __launch_bounds__(64 * DW) void attention_bf16_decode_kernel(AttnTileArgs a) {
   // per wave: maximum and sum per row, unnormalised accumulator [16][D]
   extern __shared__ float lds[];
@@ -406,22 +660,22 @@ __global__ __launch_bounds__(64 * DW) void attention_bf16_decode_kernel(AttnTile
     int pgA[3], pgB[3];
     int b = b0 + wave;
     if (b < b1) {
-      block_pages(table, b << 5, lo, pos_max, a.page_size, r16, quad, pgA);
-      block_load(a, kvh, b << 5, lo, pos_max, r16, quad, pgA, A);
+      block_pages<P2>(table, b << 5, lo, pos_max, a.page_size, r16, quad, pgA);
+      block_load<P2>(a, kvh, b << 5, lo, pos_max, r16, quad, pgA, A);
     }
-    if (b + DW < b1) block_pages(table, (b + DW) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
+    if (b + DW < b1) block_pages<P2>(table, (b + DW) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
     while (b < b1) {
       const int vpa = pgA[2];
-      if (b + DW < b1) block_load(a, kvh, (b + DW) << 5, lo, pos_max, r16, quad, pgB, B);
-      block_load_values(a, kvh, b << 5, r16, quad, vpa, v);
-      if (b + 2 * DW < b1) block_pages(table, (b + 2 * DW) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
+      if (b + DW < b1) block_load<P2>(a, kvh, (b + DW) << 5, lo, pos_max, r16, quad, pgB, B);
+      block_load_values<P2>(a, kvh, b << 5, r16, quad, vpa, v);
+      if (b + 2 * DW < b1) block_pages<P2>(table, (b + 2 * DW) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
       block_compute(A, v, qreg, qtail, b << 5, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
       b += DW;
       if (b >= b1) break;
       const int vpb = pgB[2];
-      if (b + DW < b1) block_load(a, kvh, (b + DW) << 5, lo, pos_max, r16, quad, pgA, A);
-      block_load_values(a, kvh, b << 5, r16, quad, vpb, v);
-      if (b + 2 * DW < b1) block_pages(table, (b + 2 * DW) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
+      if (b + DW < b1) block_load<P2>(a, kvh, (b + DW) << 5, lo, pos_max, r16, quad, pgA, A);
+      block_load_values<P2>(a, kvh, b << 5, r16, quad, vpb, v);
+      if (b + 2 * DW < b1) block_pages<P2>(table, (b + 2 * DW) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
       block_compute(B, v, qreg, qtail, b << 5, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
       b += DW;
     }
@@ -480,9 +734,11 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse), "attention: split run without scratch");
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
   if (a.num_tiles == 0) return 0;
+  const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
   dim3 grid(a.num_tiles, a.nkv, a.num_splits), block(64 * DW);
   const size_t smem = (size_t)(2 * DW * 16 + DW * 16 * D) * sizeof(float);
-  attention_bf16_decode_kernel<<<grid, block, smem, stream>>>(a);
+  if (p2) attention_bf16_decode_kernel<true><<<grid, block, smem, stream>>>(a);
+  else attention_bf16_decode_kernel<false><<<grid, block, smem, stream>>>(a);
   QRT_LAUNCH_CHECK("attention_bf16_decode");
   if (a.num_splits > 1) {
     attention_merge_kernel<<<dim3(num_rows_total), dim3(D >= 64 ? 64 : 32), 0, stream>>>(a.part_o, a.part_lse, a.out,
@@ -505,10 +761,22 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse), "attention: split run without scratch");
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
   if (a.num_tiles == 0) return 0;
+  const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
   dim3 grid(a.num_tiles, a.nkv, a.num_splits), block(64 * a.waves);
-  if (a.row_tiles == 1) attention_bf16_kernel<1><<<grid, block, 0, stream>>>(a);
-  else if (a.row_tiles == 2) attention_bf16_kernel<2><<<grid, block, 0, stream>>>(a);
-  else if (a.row_tiles == 4 && D <= 128) attention_bf16_kernel<4><<<grid, block, 0, stream>>>(a);
+  if (a.row_tiles == 2 && a.waves == 4 && a.num_splits == 1 && a.use_lds) {
+    const size_t smem = 2 * (size_t)STAGE_ELEMS * sizeof(bf16_t);
+    QRT_CHECK(smem <= 64 * 1024, "attention: head size %d needs %zu bytes of LDS", D, smem);
+    if (p2) attention_bf16_prefill_kernel<2, true><<<grid, block, smem, stream>>>(a);
+    else attention_bf16_prefill_kernel<2, false><<<grid, block, smem, stream>>>(a);
+    QRT_LAUNCH_CHECK("attention_bf16_prefill");
+    return 0;
+  }
+  if (a.row_tiles == 1 && p2) attention_bf16_kernel<1, true><<<grid, block, 0, stream>>>(a);
+  else if (a.row_tiles == 1) attention_bf16_kernel<1, false><<<grid, block, 0, stream>>>(a);
+  else if (a.row_tiles == 2 && p2) attention_bf16_kernel<2, true><<<grid, block, 0, stream>>>(a);
+  else if (a.row_tiles == 2) attention_bf16_kernel<2, false><<<grid, block, 0, stream>>>(a);
+  else if (a.row_tiles == 4 && D <= 128 && p2) attention_bf16_kernel<4, true><<<grid, block, 0, stream>>>(a);
+  else if (a.row_tiles == 4 && D <= 128) attention_bf16_kernel<4, false><<<grid, block, 0, stream>>>(a);
   else return qrt_fail("attention: %d row tiles per wave at head size %d is not built", a.row_tiles, D);
   QRT_LAUNCH_CHECK("attention_bf16");
   if (a.num_splits > 1) {

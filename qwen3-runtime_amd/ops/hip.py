@@ -63,7 +63,7 @@ class _AttnTileArgs(Structure):
         ("tile_seq", c_void_p), ("tile_row0", c_void_p), ("part_o", c_void_p), ("part_lse", c_void_p),
         ("table_width", c_int), ("num_tiles", c_int), ("nq", c_int), ("nkv", c_int),
         ("page_size", c_int), ("window", c_int), ("num_splits", c_int), ("waves", c_int),
-        ("scale_log2", c_float), ("row_tiles", c_int),
+        ("scale_log2", c_float), ("row_tiles", c_int), ("use_lds", c_int),
     ]
 
 
@@ -133,6 +133,8 @@ class HipOps:
     own_max_rows = 16
     # tiles of 16 rows per wave in the attention kernel for long portions (1, 2 or 4)
     prefill_row_tiles = 2
+    # long portions: keys and values go through LDS, shared by the four waves of a block
+    prefill_through_lds = True
 
     def __init__(self):
         self.lib = core_library()
@@ -435,6 +437,8 @@ class HipOps:
         return max(1, min((256 + work - 1) // work, blocks // 8, 64))
 
     def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window):
+        if not scale > 0:
+            raise OpsError(f"the bfloat16 attention kernels take a positive score scale, not {scale}")
         lib = attention_library(d)
         g = nq // nkv
         max_rows = ctx.max_q_len * g
@@ -461,6 +465,7 @@ class HipOps:
         a.tile_row0 = tiles.data_ptr() + 4 * n_tiles
         a.num_tiles, a.nq, a.nkv, a.page_size, a.window = n_tiles, nq, nkv, cache.group.page_size, window
         a.num_splits, a.waves, a.row_tiles = splits, waves, row_tiles
+        a.use_lds = 1 if self.prefill_through_lds else 0
         a.scale_log2 = scale * math.log2(math.e)
         if splits > 1:
             part_o = torch.empty((ctx.num_tokens * nq * splits, d), dtype=torch.float32, device=q.device)

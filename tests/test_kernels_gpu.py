@@ -299,6 +299,8 @@ ATTN_CASES = [
     ([(40, 200), (1, 1000)], 32, 8, 128, 16),
     ([(9, 50)], 3, 3, 80, 16),
     ([(1, 700)], 34, 2, 16, 32),
+    ([(1, 100), (2, 61), (1, 24)], 4, 2, 32, 24),   # page sizes that are no power of two
+    ([(20, 131), (300, 300)], 4, 1, 64, 40),
 ]
 
 
