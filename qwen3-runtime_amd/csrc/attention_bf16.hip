@@ -6,7 +6,7 @@
 // q_len * g rows, row = token * g + (query head within the group): all g query
 // heads that share a key head sit in the same tile, so a decoded token fills g
 // rows and a prompt portion fills tiles of 16 rows per wave. The host passes a
-// list of tiles (sequence, first row); blockIdx.x walks it.
+// list of tiles (sequence, first row); the grid walks it, one block per tile and key head.
 //
 // Products. Scores are formed transposed, S^T = K Q^T, with the 16x16x32 MFMA:
 // the A operand is 16 keys x 32 head elements read straight from the key page,
@@ -144,14 +144,16 @@ template <int RT, bool P2>
 __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(AttnTileArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int seq = a.tile_seq[blockIdx.x];
-  const int kvh = blockIdx.y, split = blockIdx.z;
+  // blocks of one tile are neighbours in the launch order, one per key head: with as many key
+  // heads as XCDs, a head's keys and values stay in one XCD's L2
+  const int tile = blockIdx.x / a.nkv, kvh = blockIdx.x - tile * a.nkv, split = blockIdx.z;
+  const int seq = a.tile_seq[tile];
   const int g = a.nq / a.nkv;
   const int q_begin = a.cu_q[seq];
   const int q_len = a.cu_q[seq + 1] - q_begin;
   const int kv_len = a.kv_lens[seq];
   const int n_rows = q_len * g;
-  const int row0 = a.tile_row0[blockIdx.x] + 16 * RT * wave;
+  const int row0 = a.tile_row0[tile] + 16 * RT * wave;
   if (row0 >= n_rows) return;
   const int first_pos = kv_len - q_len;
   const int ps = a.page_size, psh = __builtin_ctz(ps);
@@ -292,14 +294,14 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   extern __shared__ bf16_t lds_kv[];  // [2][STAGE_ELEMS]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int seq = a.tile_seq[blockIdx.x];
-  const int kvh = blockIdx.y;
+  const int tile = blockIdx.x / a.nkv, kvh = blockIdx.x - tile * a.nkv;
+  const int seq = a.tile_seq[tile];
   const int g = a.nq / a.nkv;
   const int q_begin = a.cu_q[seq];
   const int q_len = a.cu_q[seq + 1] - q_begin;
   const int kv_len = a.kv_lens[seq];
   const int n_rows = q_len * g;
-  const int tile_row0 = a.tile_row0[blockIdx.x];  // first row of the block of waves; < n_rows
+  const int tile_row0 = a.tile_row0[tile];  // first row of the block of waves; < n_rows
   const int row0 = tile_row0 + 16 * RT * wave;
   const bool wave_has_rows = row0 < n_rows;
   const int first_pos = kv_len - q_len;
@@ -517,11 +519,16 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
 // more than the second launch: measured 355 us against 98 us at 64 sequences.)
 constexpr int DW = 4;
 
-struct KvBlock {  // the keys of one block, as MFMA operands
+struct KvBlock {  // the keys and values of one block of 32 keys, as MFMA operands
   bf16x8_t k[2][KFULL > 0 ? KFULL : 1];
   bf16x8_t kt[2];
+  bf16x8_t v[DB];
 };
 
+// Every load is unconditional: positions are clamped into [lo, pos_max], which lies in pages
+// the sequence holds; what was read from a clamped place is masked (keys) or zeroed (values)
+// before use. Loads under branches would make the compiler wait for all loads in flight
+// wherever it can no longer count them.
 template <bool P2>
 __device__ __forceinline__ void block_pages(const int* __restrict__ table, int base, int lo, int pos_max, int ps,
                                             int r16, int quad, int pg[3]) {
@@ -531,14 +538,14 @@ __device__ __forceinline__ void block_pages(const int* __restrict__ table, int b
     const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
     pg[kb] = table[page_div<P2>(kidx, ps, psh)];
   }
-  const int kv0 = base + 8 * quad;
-  pg[2] = (kv0 <= pos_max && kv0 + 7 >= lo) ? table[page_div<P2>(kv0, ps, psh)] : -1;
+  const int kv0 = min(max(base + 8 * quad, lo & ~7), pos_max & ~7);
+  pg[2] = table[page_div<P2>(kv0, ps, psh)];
 }
 
 template <bool P2>
 __device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int base, int lo, int pos_max, int r16,
                                            int quad, const int pg[3], KvBlock& blk) {
-  const int ps = a.page_size, psh = __builtin_ctz(ps);
+  const int ps = a.page_size;
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
     const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
@@ -547,27 +554,14 @@ __device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int b
     for (int i = 0; i < KFULL; ++i) blk.k[kb][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
     if (KTAIL) blk.kt[kb] = load_tail(kp + 32 * KFULL, quad);
   }
+  const int kv0 = min(max(base + 8 * quad, lo & ~7), pos_max & ~7);
+  const bf16_t* vp = a.v_cache + (((size_t)pg[2] * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps);
+#pragma unroll
+  for (int i = 0; i < DB; ++i) blk.v[i] = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
 }
 
-template <bool P2>
-__device__ __forceinline__ void block_load_values(const AttnTileArgs& a, int kvh, int base, int r16, int quad,
-                                                  int vpage, bf16x8_t* v) {
-  const int ps = a.page_size, psh = __builtin_ctz(ps);
-  const int kv0 = base + 8 * quad;
-  const bool vload = vpage >= 0;
-  const bf16_t* vp = a.v_cache + (((size_t)(vload ? vpage : 0) * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps);
-#pragma unroll
-  for (int i = 0; i < DB; ++i) {
-    if (vload) v[i] = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
-    else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[i][e] = (bf16_t)0.0f;
-    }
-  }
-}
-
-__device__ __forceinline__ void block_compute(const KvBlock& blk, const bf16x8_t* v, const bf16x8_t* qreg,
-                                              bf16x8_t qtail, int base, int quad, bool row_valid, int qpos,
+__device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg, bf16x8_t qtail, int base, int lo,
+                                              int pos_min, int pos_max, int quad, bool row_valid, int qpos,
                                               int window, float scale_log2, float& m, float& l, f32x4_t* o) {
   f32x4_t s[2];
 #pragma unroll
@@ -578,39 +572,22 @@ __device__ __forceinline__ void block_compute(const KvBlock& blk, const bf16x8_t
     if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kt[kb], qtail, acc, 0, 0, 0);
     s[kb] = acc;
   }
-  float p[8];
-  float mx = -INFINITY;
+  // the same for the whole wave: does every row see all 32 keys?
+  const bool whole = base + 31 <= pos_min && (window == 0 || base > pos_max - window);
+  if (!whole) {
+    // values of keys outside [lo, pos_max] came from a clamped place and may be anything
+    const int kv0 = base + 8 * quad;
+    const bool seen = kv0 <= pos_max && kv0 + 7 >= lo;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int key = base + 8 * quad + e;
-    const bool vis = row_valid && key <= qpos && (window == 0 || key > qpos - window);
-    p[e] = vis ? s[e >> 2][e & 3] * scale_log2 : -INFINITY;
-    mx = fmaxf(mx, p[e]);
-  }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-  const float m_new = fmaxf(m, mx);
-  const float m_use = m_new == -INFINITY ? 0.f : m_new;
-  const float corr = exp2f(m - m_use);
-  float psum = 0.f;
-  bf16x8_t pb;
+    for (int i = 0; i < DB; ++i)
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float pe = exp2f(p[e] - m_use);
-    psum += pe;
-    pb[e] = (bf16_t)pe;
+      for (int e = 0; e < 8; ++e) blk.v[i][e] = seen ? blk.v[i][e] : (bf16_t)0.0f;
   }
-  l = l * corr + psum;
-  m = m_new;
-#pragma unroll
-  for (int i = 0; i < DB; ++i) {
-    o[i] *= corr;
-    o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v[i], pb, o[i], 0, 0, 0);
-  }
+  tile_update(s, blk.v, !whole, base, quad, row_valid, qpos, window, scale_log2, m, l, o);
 }
 
 template <bool P2>
-__global__ __launch_bounds__(64 * DW) void attention_bf16_decode_kernel(AttnTileArgs a) {
+__global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_decode_kernel(AttnTileArgs a) {
   // per wave: maximum and sum per row, unnormalised accumulator [16][D]
   extern __shared__ float lds[];
   float* lds_m = lds;                 // [DW][16]
@@ -639,7 +616,15 @@ __global__ __launch_bounds__(64 * DW) void attention_bf16_decode_kernel(AttnTile
   for (int i = 0; i < DB; ++i) o[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  if (n_rows > 0) {
+  const int pos_min = first_pos, pos_max = first_pos + (max(n_rows, 1) - 1) / g;
+  const int lo = a.window > 0 ? max(0, pos_min - a.window + 1) : 0;
+  const int blk_begin = lo >> 5, blk_end = (pos_max >> 5) + 1;
+  const int per = (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
+  const int b0 = blk_begin + split * per;
+  const int b1 = min(blk_end, b0 + per);
+  int b = b0 + wave;
+
+  if (n_rows > 0 && b < b1) {
     const bf16_t* qp = a.q + ((size_t)(q_begin + tok) * a.nq + head) * D;
     bf16x8_t qreg[KFULL > 0 ? KFULL : 1];
 #pragma unroll
@@ -647,37 +632,25 @@ __global__ __launch_bounds__(64 * DW) void attention_bf16_decode_kernel(AttnTile
     bf16x8_t qtail = load_tail(qp, 2);  // zeros
     if (KTAIL) qtail = load_tail(qp + 32 * KFULL, quad);
 
-    const int pos_min = first_pos, pos_max = first_pos + (n_rows - 1) / g;
-    const int lo = a.window > 0 ? max(0, pos_min - a.window + 1) : 0;
-    const int blk_begin = lo >> 5, blk_end = (pos_max >> 5) + 1;
-    const int per = (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
-    const int b0 = blk_begin + split * per;
-    const int b1 = min(blk_end, b0 + per);
-
-    // keys are loaded one block ahead, page numbers two; values at the top of their block
+    // keys and values are loaded one block ahead, page numbers two; past the wave's last block
+    // the loads repeat that block (their data is not used)
+    const int last = b + (b1 - 1 - b) / DW * DW;
     KvBlock A, B;
-    bf16x8_t v[DB];
     int pgA[3], pgB[3];
-    int b = b0 + wave;
-    if (b < b1) {
-      block_pages<P2>(table, b << 5, lo, pos_max, a.page_size, r16, quad, pgA);
-      block_load<P2>(a, kvh, b << 5, lo, pos_max, r16, quad, pgA, A);
-    }
-    if (b + DW < b1) block_pages<P2>(table, (b + DW) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
-    while (b < b1) {
-      const int vpa = pgA[2];
-      if (b + DW < b1) block_load<P2>(a, kvh, (b + DW) << 5, lo, pos_max, r16, quad, pgB, B);
-      block_load_values<P2>(a, kvh, b << 5, r16, quad, vpa, v);
-      if (b + 2 * DW < b1) block_pages<P2>(table, (b + 2 * DW) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
-      block_compute(A, v, qreg, qtail, b << 5, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+    block_pages<P2>(table, b << 5, lo, pos_max, a.page_size, r16, quad, pgA);
+    block_pages<P2>(table, min(b + DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
+    block_load<P2>(a, kvh, b << 5, lo, pos_max, r16, quad, pgA, A);
+    while (true) {
+      block_load<P2>(a, kvh, min(b + DW, last) << 5, lo, pos_max, r16, quad, pgB, B);
+      block_pages<P2>(table, min(b + 2 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
+      block_compute(A, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
       b += DW;
       if (b >= b1) break;
-      const int vpb = pgB[2];
-      if (b + DW < b1) block_load<P2>(a, kvh, (b + DW) << 5, lo, pos_max, r16, quad, pgA, A);
-      block_load_values<P2>(a, kvh, b << 5, r16, quad, vpb, v);
-      if (b + 2 * DW < b1) block_pages<P2>(table, (b + 2 * DW) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
-      block_compute(B, v, qreg, qtail, b << 5, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+      block_load<P2>(a, kvh, min(b + DW, last) << 5, lo, pos_max, r16, quad, pgA, A);
+      block_pages<P2>(table, min(b + 2 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
+      block_compute(B, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
       b += DW;
+      if (b >= b1) break;
     }
   }
   l += __shfl_xor(l, 16, 64);
@@ -762,7 +735,8 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
   if (a.num_tiles == 0) return 0;
   const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
-  dim3 grid(a.num_tiles, a.nkv, a.num_splits), block(64 * a.waves);
+  QRT_CHECK((long long)a.num_tiles * a.nkv < (1ll << 31), "attention: %d tiles x %d key heads is too many blocks", a.num_tiles, a.nkv);
+  dim3 grid(a.num_tiles * a.nkv, 1, a.num_splits), block(64 * a.waves);
   if (a.row_tiles == 2 && a.waves == 4 && a.num_splits == 1 && a.use_lds) {
     const size_t smem = 2 * (size_t)STAGE_ELEMS * sizeof(bf16_t);
     QRT_CHECK(smem <= 64 * 1024, "attention: head size %d needs %zu bytes of LDS", D, smem);

@@ -404,12 +404,18 @@ class HipOps:
             self._check(self.lib, self.lib.qrt_attention_f32(byref(a), _CODE[q.dtype], _stream()))
         return out
 
+    resident_blocks = 512  # blocks of the prompt kernels the chip holds at once: 2 on each of 256 CUs
+
     @staticmethod
-    def plan_tiles(q_lens, kv_lens, group_size: int, rows_per_tile: int):
+    def plan_tiles(q_lens, kv_lens, group_size: int, rows_per_tile: int, nkv: int = 1, resident: int = 0):
         """Work list of the MFMA attention kernels: (sequence, first row) per tile of rows.
 
         Tiles that see the most keys come first: blocks that start late are then the short ones,
-        and the chip stays full until the end although causal tiles differ in length."""
+        and the chip stays full until the end although causal tiles differ in length. When all
+        blocks (tiles x ``nkv`` key heads) fit on the chip at once (``resident``), nothing starts
+        late: each CU then holds block i and block i + resident / 2 of the launch order from start
+        to end, so the second half of the list is turned round and long tiles share a CU with
+        short ones."""
         items = []
         for s, (n, kv) in enumerate(zip(q_lens, kv_lens)):
             first = kv - n
@@ -417,6 +423,9 @@ class HipOps:
                 last_tok = min(n * group_size, r + rows_per_tile) - 1
                 items.append((-(first + last_tok // group_size), s, r))
         items.sort()
+        half = resident // (2 * max(nkv, 1))
+        if resident and half < len(items) <= 2 * half:
+            items = items[:half] + items[half:][::-1]
         seqs = [s for _, s, _ in items]
         row0 = [r for _, _, r in items]
         return np.asarray(seqs + row0, dtype=np.int32), len(seqs)
@@ -449,7 +458,8 @@ class HipOps:
         key = ("attn_tiles", g, waves, row_tiles)
         plan = ctx.scratch.get(key)
         if plan is None:
-            host, n_tiles = self.plan_tiles(ctx.q_lens_host, ctx.kv_lens_host, g, 16 * waves * row_tiles)
+            host, n_tiles = self.plan_tiles(ctx.q_lens_host, ctx.kv_lens_host, g, 16 * waves * row_tiles, nkv,
+                                            self.resident_blocks if waves == 4 and row_tiles >= 2 else 0)
             plan = (torch.from_numpy(host).to(q.device), n_tiles)
             ctx.scratch[key] = plan
         tiles, n_tiles = plan
