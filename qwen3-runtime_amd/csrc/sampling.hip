@@ -119,25 +119,57 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   const bool keep = !greedy || a.write_work;
   float m = -INFINITY, ssum = 0.f;
   int bi = 0x7fffffff;
-#pragma unroll 4
-  for (int i = tid; i < V; i += blockDim.x) {
-    float v = lg[i];
-    if (cnt) {
-      const int c = cnt[i];
-      if (c > 0) {
-        v = v > 0.f ? v / rep : v * rep;
-        v -= pres;
-        v -= freq * (float)c;
-      }
+  auto take = [&](float v, int c, int i) -> float {  // processed value of id i; updates m, ssum, bi
+    if (c > 0) {
+      v = v > 0.f ? v / rep : v * rep;
+      v -= pres;
+      v -= freq * (float)c;
     }
     if (!greedy) v = v / temp;
-    if (keep) x[i] = v;
     if (v > m) {
       ssum = ssum * expf(m - v) + 1.0f;  // m = -inf at first: exp(-inf) = 0
       m = v;
       bi = i;
     } else if (v == v) {
       ssum += expf(v - m);
+    }
+    return v;
+  };
+  if ((V & 3) == 0) {
+    // rows start on 16-byte boundaries: four ids per load, several loads in flight per thread
+    // (one block reads the whole row, so the time is the memory's latency times the number of
+    // rounds of loads)
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    constexpr int U = 6;
+    const int V4 = V >> 2;
+    for (int i0 = tid; i0 < V4; i0 += U * blockDim.x) {
+      f32x4 v[U];
+      i32x4 c[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + u * blockDim.x;
+        if (i < V4) {
+          v[u] = ((const f32x4*)lg)[i];
+          c[u] = cnt ? ((const i32x4*)cnt)[i] : (i32x4){0, 0, 0, 0};
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + u * blockDim.x;
+        if (i < V4) {
+          f32x4 w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = take(v[u][e], c[u][e], 4 * i + e);
+          if (keep) ((f32x4*)x)[i] = w;
+        }
+      }
+    }
+  } else {
+#pragma unroll 4
+    for (int i = tid; i < V; i += blockDim.x) {
+      const float v = take(lg[i], cnt ? cnt[i] : 0, i);
+      if (keep) x[i] = v;
     }
   }
   // merge over the wave, then over the block: the larger maximum wins, ties go to the lower index
