@@ -331,6 +331,135 @@ __global__ void qk_norm_rope_store_kernel(QkArgs a) {
   }
 }
 
+// The same work for head sizes 16, 32, ..., 512 (powers of two) with every access 8 elements
+// wide. Norm and rotation: a lane owns 8 neighbouring elements of the first half of a head and
+// their partners in the second half, head_dim / 16 lanes share a head, a wave covers
+// 64 / (head_dim / 16) heads per pass and computes the sines and cosines of its token once for
+// all passes it makes. Values: a wave takes 8 tokens of one head, turns them round in LDS and
+// writes, for each head element, the 8 tokens as one piece of the transposed page; that needs
+// the 8 slots to be neighbours that start on a multiple of 8, as the tokens of a prompt
+// portion usually are, otherwise it writes element by element.
+template <typename T> struct alignas(sizeof(T) * 8) Vec8 { T v[8]; };
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_rope_store_wide_kernel(QkArgs a, int lph, int rope_blocks,
+                                                                      int passes_per_wave) {
+  extern __shared__ __align__(32) unsigned char smem_raw[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int D = a.head_dim, half = D >> 1;
+
+  if ((int)blockIdx.x < rope_blocks) {
+    const int hp = 64 / lph, nh = a.nq + a.nkv;
+    const int passes = (nh + hp - 1) / hp;
+    const int groups = (passes + passes_per_wave - 1) / passes_per_wave;
+    const long item = (long)blockIdx.x * 4 + wave;
+    if (item >= (long)a.num_tokens * groups) return;
+    const int t = (int)(item / groups), grp = (int)(item - (long)t * groups);
+    const int c = lane & (lph - 1), hl = lane / lph;
+    float sn[8], cs[8];
+    if (a.inv_freq) {
+      const float pos = (float)a.positions[t];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sincosf(pos * a.inv_freq[8 * c + e], &sn[e], &cs[e]);
+    }
+    const int slot = a.slots ? a.slots[t] : 0;
+    const int page = slot / a.page_size, off = slot - page * a.page_size;
+    const int pass_end = min(passes, (grp + 1) * passes_per_wave);
+    for (int ps = grp * passes_per_wave; ps < pass_end; ++ps) {
+      const int h = ps * hp + hl;
+      if (h >= nh) continue;  // whole groups of lph lanes leave together
+      const bool is_q = h < a.nq;
+      const int hh = is_q ? h : h - a.nq;
+      const T* src = is_q ? (const T*)a.q_in + (size_t)t * a.q_stride + (size_t)hh * D
+                          : (const T*)a.k_in + (size_t)t * a.k_stride + (size_t)hh * D;
+      const float* w = is_q ? a.q_weight : a.k_weight;
+      const Vec8<T> r1 = *(const Vec8<T>*)(src + 8 * c), r2 = *(const Vec8<T>*)(src + half + 8 * c);
+      float x1[8], x2[8];
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        x1[e] = to_f32<T>(r1.v[e]);
+        x2[e] = to_f32<T>(r2.v[e]);
+        ss += x1[e] * x1[e] + x2[e] * x2[e];
+      }
+      if (w) {
+        for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        const float inv = rsqrtf(ss / (float)D + a.eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          x1[e] = x1[e] * inv * w[8 * c + e];
+          x2[e] = x2[e] * inv * w[half + 8 * c + e];
+        }
+      }
+      Vec8<T> y1, y2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float u1 = x1[e], u2 = x2[e];
+        if (a.inv_freq) {
+          u1 = x1[e] * cs[e] - x2[e] * sn[e];
+          u2 = x2[e] * cs[e] + x1[e] * sn[e];
+        }
+        y1.v[e] = from_f32<T>(u1);
+        y2.v[e] = from_f32<T>(u2);
+      }
+      T* dense = nullptr;
+      if (is_q && a.q_out) dense = (T*)a.q_out + ((size_t)t * a.nq + hh) * D;
+      if (!is_q && a.k_out) dense = (T*)a.k_out + ((size_t)t * a.nkv + hh) * D;
+      if (dense) {
+        *(Vec8<T>*)(dense + 8 * c) = y1;
+        *(Vec8<T>*)(dense + half + 8 * c) = y2;
+      }
+      if (!is_q && a.slots) {
+        T* paged = (T*)a.k_cache + (((size_t)page * a.nkv + hh) * a.page_size + off) * D;
+        *(Vec8<T>*)(paged + 8 * c) = y1;
+        *(Vec8<T>*)(paged + half + 8 * c) = y2;
+      }
+    }
+    return;
+  }
+
+  // values: 8 tokens of one head
+  const long item = (long)(blockIdx.x - rope_blocks) * 4 + wave;
+  const int token_groups = (a.num_tokens + 7) >> 3;
+  if (item >= (long)token_groups * a.nv) return;
+  const int tg = (int)(item / a.nv), hv = (int)(item - (long)tg * a.nv);
+  const int t0 = 8 * tg, nvalid = min(8, a.num_tokens - t0);
+  const int row = D + 8;  // padded: the 8 tokens of an element lie in different banks
+  T* tile = (T*)smem_raw + (size_t)wave * 8 * row;
+  const int chunks = D >> 3;
+  for (int idx = lane; idx < 8 * chunks; idx += 64) {
+    const int j = idx / chunks, c = idx - j * chunks;
+    if (j < nvalid) {
+      const Vec8<T> r = *(const Vec8<T>*)((const T*)a.v_in + (size_t)(t0 + j) * a.v_stride + (size_t)hv * D + 8 * c);
+      *(Vec8<T>*)(tile + j * row + 8 * c) = r;
+      if (a.v_out) *(Vec8<T>*)((T*)a.v_out + ((size_t)(t0 + j) * a.nv + hv) * D + 8 * c) = r;
+    }
+  }
+  if (!a.slots) return;
+  __builtin_amdgcn_wave_barrier();  // the wave reads below what it wrote above; LDS keeps a wave's order
+  const int my_slot = a.slots[t0 + min(lane, nvalid - 1)];
+  const int s0 = __shfl(my_slot, 0, 64);
+  const bool in_line = lane >= 8 || my_slot == s0 + lane;
+  const bool wide = nvalid == 8 && (s0 & 7) == 0 && (a.page_size & 7) == 0 && __all(in_line);
+  if (wide) {
+    const int page = s0 / a.page_size, off = s0 - page * a.page_size;
+    T* base = (T*)a.v_cache + ((size_t)page * a.nv + hv) * D * a.page_size + off;
+    for (int d = lane; d < D; d += 64) {
+      Vec8<T> o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o.v[j] = tile[j * row + d];
+      *(Vec8<T>*)(base + (size_t)d * a.page_size) = o;
+    }
+  } else {
+    for (int j = 0; j < nvalid; ++j) {
+      const int sj = __shfl(my_slot, j, 64);
+      const int page = sj / a.page_size, off = sj - page * a.page_size;
+      T* base = (T*)a.v_cache + ((size_t)page * a.nv + hv) * D * a.page_size + off;
+      for (int d = lane; d < D; d += 64) base[(size_t)d * a.page_size] = tile[j * row + d];
+    }
+  }
+}
+
 extern "C" int qrt_qk_norm_rope_store(const QkArgs* args, int dtype, long num_cache_pages, hipStream_t stream) {
   QkArgs a = *args;
   QRT_CHECK(a.num_tokens >= 0 && a.nq >= 0 && a.nkv >= 0 && a.nv >= 0, "qk_norm_rope_store: negative size");
@@ -348,6 +477,33 @@ extern "C" int qrt_qk_norm_rope_store(const QkArgs* args, int dtype, long num_ca
   const long items = (long)a.num_tokens * (a.nq + a.nkv + a.nv);
   if (items == 0) return 0;
   const int waves = 4;
+  const size_t esize = dtype == QRT_F32 ? 4 : 2;
+  auto lined_up = [&](const void* ptr) { return ((uintptr_t)ptr % (8 * esize)) == 0; };
+  const int D = a.head_dim;
+  const bool wide = D >= 16 && (D & (D - 1)) == 0 && a.q_stride % 8 == 0 && a.k_stride % 8 == 0 &&
+                    a.v_stride % 8 == 0 && lined_up(a.q_in) && lined_up(a.k_in) && lined_up(a.v_in) &&
+                    lined_up(a.q_out) && lined_up(a.k_out) && lined_up(a.v_out) && lined_up(a.k_cache) &&
+                    lined_up(a.v_cache);
+  if (wide) {
+    const int lph = D / 16, hp = 64 / lph, nh = a.nq + a.nkv;
+    const int passes = (nh + hp - 1) / hp;
+    // many tokens: a wave makes all passes of its token and computes its sines and cosines once
+    const int ppw = (long)a.num_tokens * passes >= 4096 ? (passes > 0 ? passes : 1) : 1;
+    const int groups = passes > 0 ? (passes + ppw - 1) / ppw : 0;
+    const long rope_items = (long)a.num_tokens * groups;
+    const long v_items = (long)((a.num_tokens + 7) / 8) * a.nv;
+    const long rope_blocks = (rope_items + waves - 1) / waves, v_blocks = (v_items + waves - 1) / waves;
+    QRT_CHECK(rope_blocks + v_blocks < (1l << 31), "qk_norm_rope_store: too many tokens");
+    dim3 grid((unsigned)(rope_blocks + v_blocks)), block(64 * waves);
+    const size_t smem = (size_t)waves * 8 * (D + 8) * esize;
+    if (dtype == QRT_F32)
+      qk_norm_rope_store_wide_kernel<float><<<grid, block, smem, stream>>>(a, lph, (int)rope_blocks, ppw);
+    else if (dtype == QRT_BF16)
+      qk_norm_rope_store_wide_kernel<bf16_t><<<grid, block, smem, stream>>>(a, lph, (int)rope_blocks, ppw);
+    else return qrt_fail("qk_norm_rope_store: unknown dtype %d", dtype);
+    QRT_LAUNCH_CHECK("qk_norm_rope_store (wide)");
+    return 0;
+  }
   dim3 grid((unsigned)((items + waves - 1) / waves)), block(64 * waves);
   if (dtype == QRT_F32) qk_norm_rope_store_kernel<float><<<grid, block, 0, stream>>>(a);
   else if (dtype == QRT_BF16) qk_norm_rope_store_kernel<bf16_t><<<grid, block, 0, stream>>>(a);

@@ -249,6 +249,32 @@ def test_qk_norm_rope_store(ops, dtype, nq, nkv, d, ps, theta):
     close(cache2.v, want_cache.v, 0, 0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("t,nq,nkv,d,ps,start", [(40, 6, 2, 32, 8, 16), (37, 4, 2, 64, 16, 8), (21, 4, 2, 16, 8, 3),
+                                                 (700, 32, 8, 128, 16, 0), (9, 3, 1, 48, 8, 0)])
+def test_qk_norm_rope_store_neighbouring_slots(ops, dtype, t, nq, nkv, d, ps, start):
+    """A prompt portion: consecutive positions in consecutive slots, so that values go into their
+    transposed pages eight tokens at a time (where the run starts on a multiple of eight) or one
+    by one (start 3, and the tail of every run); with 700 tokens a wave makes all passes over the
+    heads of its token."""
+    pages = (start + t + ps - 1) // ps + 2
+    qkv = rnd(t, (nq + 2 * nkv) * d, dtype=dtype)
+    qw, kw = 1 + 0.1 * rnd(d, seed=5), 1 + 0.1 * rnd(d, seed=6)
+    inv = (1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    pos = torch.arange(start, start + t, dtype=torch.int32, device=DEV)
+    order = torch.randperm(pages)
+    slots = torch.tensor([int(order[p // ps]) * ps + p % ps for p in range(start, start + t)], dtype=torch.int32, device=DEV)
+    cache = make_cache(pages, nkv, ps, d, dtype)
+    cache.group.slots = slots
+    want_cache = make_cache(pages, nkv, ps, d, dtype)
+    want = R.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, pos, want_cache.k, want_cache.v, slots, ps)
+    got = ops.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, pos, cache)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    close(got, want, tol, tol)
+    close(cache.k, want_cache.k, tol, tol)
+    close(cache.v, want_cache.v, 0, 0)
+
+
 def build_attention_case(seqs, nq, nkv, d, ps, dtype, seed=0, window=None, shuffle=True, spare_pages=3):
     """seqs: list of (q_len, kv_len). Returns q, cache view with filled pages, ctx."""
     from qwen3_runtime_amd.parts.base import StepContext
