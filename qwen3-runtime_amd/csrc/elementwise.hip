@@ -480,7 +480,9 @@ extern "C" int qrt_qk_norm_rope_store(const QkArgs* args, int dtype, long num_ca
   const size_t esize = dtype == QRT_F32 ? 4 : 2;
   auto lined_up = [&](const void* ptr) { return ((uintptr_t)ptr % (8 * esize)) == 0; };
   const int D = a.head_dim;
-  const bool wide = D >= 16 && (D & (D - 1)) == 0 && a.q_stride % 8 == 0 && a.k_stride % 8 == 0 &&
+  // few tokens (decoding): the time is the launch and one round of memory latency, and the
+  // one-head-per-wave kernel has the shorter chain
+  const bool wide = a.num_tokens >= 32 && D >= 16 && (D & (D - 1)) == 0 && a.q_stride % 8 == 0 && a.k_stride % 8 == 0 &&
                     a.v_stride % 8 == 0 && lined_up(a.q_in) && lined_up(a.k_in) && lined_up(a.v_in) &&
                     lined_up(a.q_out) && lined_up(a.k_out) && lined_up(a.v_out) && lined_up(a.k_cache) &&
                     lined_up(a.v_cache);

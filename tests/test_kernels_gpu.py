@@ -250,7 +250,7 @@ def test_qk_norm_rope_store(ops, dtype, nq, nkv, d, ps, theta):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("t,nq,nkv,d,ps,start", [(40, 6, 2, 32, 8, 16), (37, 4, 2, 64, 16, 8), (21, 4, 2, 16, 8, 3),
+@pytest.mark.parametrize("t,nq,nkv,d,ps,start", [(40, 6, 2, 32, 8, 16), (37, 4, 2, 64, 16, 8), (33, 4, 2, 16, 8, 3),
                                                  (700, 32, 8, 128, 16, 0), (9, 3, 1, 48, 8, 0)])
 def test_qk_norm_rope_store_neighbouring_slots(ops, dtype, t, nq, nkv, d, ps, start):
     """A prompt portion: consecutive positions in consecutive slots, so that values go into their
