@@ -1,0 +1,97 @@
+"""The engine at the layer sizes of the 4B and 8B models (two layers, a small vocabulary)
+against the plain implementation: the kernels' production paths (few-row products on
+tile-major weights with K cut into planes, the gated epilogue, decode attention at head size
+128 with four query heads per key head, prompt attention through LDS, the vendor products for
+long portions) as parts of a whole model, in float32 and bfloat16."""
+
+import dataclasses
+
+import pytest
+import torch
+
+import traces
+
+pytestmark = pytest.mark.gpu
+
+# float32: the longest sums have 12,288 terms instead of the tiny models' few hundred.
+TOL_F32 = dict(atol=2e-4, rtol=2e-4)
+
+
+def check_rounding_noise(got, want):
+    """bfloat16 against the float32 plain implementation. Activations are rounded to 8 bits of
+    mantissa some seven times per layer, which leaves an error that behaves like noise: measured
+    at both sizes and under every cutting, its root mean square is 1.0 % of the logits' standard
+    deviation and its largest value five times that (what 400,000 Gaussian samples give). The
+    bounds leave half as much again; a fault in a page, a mask or a portion's edge moves logits
+    by a sizeable part of their standard deviation."""
+    keys = sorted(want)
+    assert set(got) == set(want)
+    w = torch.stack([want[k].double() for k in keys])
+    err = torch.stack([got[k].double() for k in keys]) - w
+    std = float(w.std())
+    rms = float(err.pow(2).mean().sqrt())
+    worst = float(err.abs().max())
+    where = keys[int(err.abs().amax(dim=1).argmax())]
+    assert rms < 0.015 * std, f"rms error {rms:.4f} against a logit deviation of {std:.3f}"
+    assert worst < 0.08 * std, f"largest error {worst:.4f} at (request, position) {where}; logit deviation {std:.3f}"
+
+
+@pytest.fixture(scope="module")
+def sized_folders(tmp_path_factory):
+    from qwen3_runtime_amd.config.presets import preset
+    from qwen3_runtime_amd.weights import write_model_folder
+
+    out = {}
+    for i, name in enumerate(("qwen3_4b", "qwen3_8b")):
+        cfg = dataclasses.replace(preset(name), num_hidden_layers=2, vocab_size=2048, eos_token_id=None)
+        folder = tmp_path_factory.mktemp(name)
+        write_model_folder(folder, cfg.to_dict(), seed=21 + i)
+        out[name] = (cfg, folder)
+    return out
+
+
+@pytest.fixture(scope="module")
+def plain_results(sized_folders):
+    out = {}
+    for name, (cfg, folder) in sized_folders.items():
+        reqs = traces.make_requests(cfg.vocab_size, [150, 41, 9], seed=6)
+        out[name] = (reqs, traces.plain_logits(folder, reqs))
+    return out
+
+
+@pytest.mark.parametrize("dtype,cut", [("float32", "portions"), ("bfloat16", "mixed"), ("bfloat16", "tail_one_by_one")])
+@pytest.mark.parametrize("name", ["qwen3_4b", "qwen3_8b"])
+def test_model_sized_layers_match_plain(sized_folders, plain_results, name, dtype, cut):
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg, folder = sized_folders[name]
+    reqs, want = plain_results[name]
+    steps = getattr(traces, cut)(reqs)
+    page = 16
+    engine_cfg = EngineConfig(page_size=page, num_pages=traces.peak_tokens(steps) // page, max_num_seqs=4, dtype=dtype,
+                              device="cuda:0", hip_graph=False)
+    loaded = load(folder, engine_cfg)
+    got = traces.replay(loaded, steps)
+    if dtype == "float32":
+        traces.compare(got, want, **TOL_F32)
+    else:
+        check_rounding_noise(got, want)
+
+
+def test_model_sized_decode_graph_equals_eager(sized_folders):
+    """Greedy tokens of three requests at the 4B layer sizes: replayed HIP graphs give the tokens
+    of eager steps."""
+    from qwen3_runtime_amd.llm import LLM
+    from qwen3_runtime_amd.sampling import SamplingParams
+
+    cfg, folder = sized_folders["qwen3_4b"]
+    prompts = list(traces.make_requests(cfg.vocab_size, [70, 20, 5], seed=8).values())
+    outs = []
+    for graph in (False, True):
+        llm = LLM(str(folder), dtype="bfloat16", max_num_seqs=4, max_num_batched_tokens=64, block_size=16,
+                  num_kv_blocks=64, cuda_graph=graph)
+        outs.append(llm.generate(prompts, SamplingParams(temperature=0.0), max_tokens=24))
+        del llm
+        torch.cuda.empty_cache()
+    assert outs[0] == outs[1]
