@@ -62,12 +62,15 @@ def main() -> int:
     steps, warmup = args.steps, args.warmup
     page = 16
     max_batch = args.batch if (args.no_points or args.prefill_only) else max(args.batch, 64)
-    per_req_tokens = args.prompt_len + steps + warmup + max_batch + 10
+    budget = 2048  # tokens per step
+    # a request decodes while later ones are still read in: up to this many steps before the timed ones
+    lead = lambda batch: batch * -(-args.prompt_len // budget)
+    per_req_tokens = args.prompt_len + steps + warmup + lead(max_batch) + 10
     pages = max_batch * (-(-per_req_tokens // page) + 1)
     t0 = time.time()
     engine = build_engine(
         None, config=cfg, seed=20260825, dtype=args.dtype, block_size=page, num_kv_blocks=pages,
-        max_num_seqs=max_batch, max_num_batched_tokens=2048, max_model_len=args.context,
+        max_num_seqs=max_batch, max_num_batched_tokens=budget, max_model_len=args.context,
         cuda_graph=not args.no_graph,
     )
     print(f"[bench] model on device in {time.time() - t0:.1f} s, {engine.loaded.weight_bytes / 1e9:.2f} GB of weights",
@@ -79,7 +82,7 @@ def main() -> int:
     def decode_run(batch: int, k: int, w: int):
         """Prefill ``batch`` prompts, then time ``k`` decode steps after ``w`` warm-up steps."""
         prompts = torch.randint(0, cfg.vocab_size, (batch, args.prompt_len), generator=gen).tolist()
-        reqs = [engine.request(engine.add_request(p, max_tokens=k + w + batch + 8, sampling=SamplingParams()))
+        reqs = [engine.request(engine.add_request(p, max_tokens=k + w + lead(batch) + 8, sampling=SamplingParams()))
                 for p in prompts]
         while any(len(r.token_ids) == r.num_prompt_tokens for r in reqs):
             engine.step()  # prompt portions until every request has its first token
@@ -179,7 +182,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
-    if args.preset == "qwen3_4b" and args.batch == 8:
+    if args.preset == "qwen3_4b" and args.batch == 8 and args.prompt_len == 2048:
         line["vs_reference_rtx4090_batch8"] = round(value / REFERENCE_4090_B8_TOK_S, 2)
     if prefill is not None:
         line["prefill"] = prefill
