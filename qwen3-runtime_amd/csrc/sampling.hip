@@ -1,4 +1,5 @@
-// Sampling on the device: one block per row of float32 logits.
+// Sampling on the device: one block per row of float32 logits (with few rows, the first
+// pass over a row is spread over several blocks).
 //
 // Chain, in the order the reference runs it (qwen3_runtime/sampling.py:120-135):
 // penalties from per-slot counts, (greedy: first maximal id), temperature,
@@ -97,35 +98,43 @@ struct SampleArgs {
   float* out_logprob;       // [R]
   int rows, vocab;
   int write_work;           // also keep the processed logits of greedy rows
+  float* partials;          // [R, parts, 4]: maximum, sum of exp(value - maximum), first index of the maximum
+  int parts;                // > 0: the first pass ran in sample_first_pass_kernel, `parts` blocks per row
 };
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
-  __shared__ float red[32];
-  __shared__ int redi[32];
-  __shared__ float part[SAMPLE_THREADS];
-  const int r = blockIdx.x, V = a.vocab, tid = threadIdx.x;
-  const float* lg = a.logits + (size_t)r * V;
-  float* x = a.work + (size_t)r * V;
+// The first pass over ids [lo, hi) of a row: penalties (reference:
+// qwen3_runtime/sampling.py:63-71) and temperature give the processed value (written to the
+// work row if asked); alongside, a running maximum, the first index that reaches it, and the
+// sum of exp(value - maximum). lo and hi are multiples of 4 (or hi = V).
+struct RowOptions {
+  float temp, rep, pres, freq;
+  const int* cnt;  // the slot's counts, or null when no penalty is set
+  bool greedy, keep;
+};
+
+__device__ __forceinline__ RowOptions row_options(const SampleArgs& a, int r) {
   const int sl = a.slot[r];
   const float* fp = a.fparams + (size_t)sl * 8;
-  const float temp = fp[0], topp = fp[1], minp = fp[2], rep = fp[3], pres = fp[4], freq = fp[5];
+  RowOptions o;
+  o.temp = fp[0]; o.rep = fp[3]; o.pres = fp[4]; o.freq = fp[5];
+  const bool pen = a.counts && (o.rep != 1.0f || o.pres != 0.0f || o.freq != 0.0f);
+  o.cnt = pen ? a.counts + (size_t)sl * a.vocab : nullptr;
+  o.greedy = o.temp <= 0.f;
+  o.keep = !o.greedy || a.write_work;
+  return o;
+}
 
-  // one pass: penalties (reference: qwen3_runtime/sampling.py:63-71) and temperature give the
-  // processed value; alongside, a running maximum, the first index that reaches it, and the sum
-  // of exp(value - maximum)
-  const bool pen = a.counts && (rep != 1.0f || pres != 0.0f || freq != 0.0f);
-  const int* cnt = pen ? a.counts + (size_t)sl * V : nullptr;
-  const bool greedy = temp <= 0.f;
-  const bool keep = !greedy || a.write_work;
-  float m = -INFINITY, ssum = 0.f;
-  int bi = 0x7fffffff;
+__device__ __forceinline__ void first_pass(const RowOptions& o, const float* __restrict__ lg, float* __restrict__ x,
+                                           int lo, int hi, int V, float& m, float& ssum, int& bi) {
+  const int* cnt = o.cnt;
+  const int tid = threadIdx.x;
   auto take = [&](float v, int c, int i) -> float {  // processed value of id i; updates m, ssum, bi
     if (c > 0) {
-      v = v > 0.f ? v / rep : v * rep;
-      v -= pres;
-      v -= freq * (float)c;
+      v = v > 0.f ? v / o.rep : v * o.rep;
+      v -= o.pres;
+      v -= o.freq * (float)c;
     }
-    if (!greedy) v = v / temp;
+    if (!o.greedy) v = v / o.temp;
     if (v > m) {
       ssum = ssum * expf(m - v) + 1.0f;  // m = -inf at first: exp(-inf) = 0
       m = v;
@@ -137,19 +146,17 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   };
   if ((V & 3) == 0) {
     // rows start on 16-byte boundaries: four ids per load, several loads in flight per thread
-    // (one block reads the whole row, so the time is the memory's latency times the number of
-    // rounds of loads)
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     typedef int i32x4 __attribute__((ext_vector_type(4)));
     constexpr int U = 6;
-    const int V4 = V >> 2;
-    for (int i0 = tid; i0 < V4; i0 += U * blockDim.x) {
+    const int lo4 = lo >> 2, hi4 = hi >> 2;
+    for (int i0 = lo4 + tid; i0 < hi4; i0 += U * blockDim.x) {
       f32x4 v[U];
       i32x4 c[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int i = i0 + u * blockDim.x;
-        if (i < V4) {
+        if (i < hi4) {
           v[u] = ((const f32x4*)lg)[i];
           c[u] = cnt ? ((const i32x4*)cnt)[i] : (i32x4){0, 0, 0, 0};
         }
@@ -157,53 +164,101 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int i = i0 + u * blockDim.x;
-        if (i < V4) {
+        if (i < hi4) {
           f32x4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = take(v[u][e], c[u][e], 4 * i + e);
-          if (keep) ((f32x4*)x)[i] = w;
+          if (o.keep) ((f32x4*)x)[i] = w;
         }
       }
     }
   } else {
 #pragma unroll 4
-    for (int i = tid; i < V; i += blockDim.x) {
+    for (int i = lo + tid; i < hi; i += blockDim.x) {
       const float v = take(lg[i], cnt ? cnt[i] : 0, i);
-      if (keep) x[i] = v;
+      if (o.keep) x[i] = v;
     }
   }
-  // merge over the wave, then over the block: the larger maximum wins, ties go to the lower index
+}
+
+// (maximum, sum, index) of two parts of a row: the larger maximum wins, ties go to the lower index
+__device__ __forceinline__ void merge_parts(float& m, float& ssum, int& bi, float om, float os, int oi) {
+  const float mm = fmaxf(m, om);
+  const float f1 = m == -INFINITY ? 0.f : expf(m - mm), f2 = om == -INFINITY ? 0.f : expf(om - mm);
+  ssum = ssum * f1 + os * f2;
+  if (om > m || (om == m && oi < bi)) bi = oi;
+  m = mm;
+}
+
+// wave, then block: every thread leaves with the block's values in red[24], red[25], redi[24]
+__device__ __forceinline__ void block_merge(float m, float ssum, int bi, float* red, float* part, int* redi) {
+  const int tid = threadIdx.x;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     const float om = __shfl_xor(m, o, 64), os = __shfl_xor(ssum, o, 64);
     const int oi = __shfl_xor(bi, o, 64);
-    const float mm = fmaxf(m, om);
-    const float f1 = m == -INFINITY ? 0.f : expf(m - mm), f2 = om == -INFINITY ? 0.f : expf(om - mm);
-    ssum = ssum * f1 + os * f2;
-    if (om > m || (om == m && oi < bi)) bi = oi;
-    m = mm;
+    merge_parts(m, ssum, bi, om, os, oi);
   }
-  {
-    const int lane = tid & 63, wave = tid >> 6, nw = (blockDim.x + 63) >> 6;
-    if (lane == 0) { red[wave] = m; part[wave] = ssum; redi[wave] = bi; }
-    __syncthreads();
-    if (tid == 0) {
-      float mm = red[0], ss = part[0];
-      int ii = redi[0];
-      for (int w = 1; w < nw; ++w) {
-        const float om = red[w], os = part[w];
-        const int oi = redi[w];
-        const float nm = fmaxf(mm, om);
-        const float f1 = mm == -INFINITY ? 0.f : expf(mm - nm), f2 = om == -INFINITY ? 0.f : expf(om - nm);
-        ss = ss * f1 + os * f2;
-        if (om > mm || (om == mm && oi < ii)) ii = oi;
-        mm = nm;
-      }
-      if (ii == 0x7fffffff) ii = 0;  // a row of NaNs
-      red[24] = mm; red[25] = ss; redi[24] = ii;
+  const int lane = tid & 63, wave = tid >> 6, nw = (blockDim.x + 63) >> 6;
+  if (lane == 0) { red[wave] = m; part[wave] = ssum; redi[wave] = bi; }
+  __syncthreads();
+  if (tid == 0) {
+    float mm = red[0], ss = part[0];
+    int ii = redi[0];
+    for (int w = 1; w < nw; ++w) merge_parts(mm, ss, ii, red[w], part[w], redi[w]);
+    red[24] = mm; red[25] = ss; redi[24] = ii;
+  }
+  __syncthreads();
+}
+
+// With few rows one block per row would leave the chip idle while it reads the whole
+// vocabulary: the first pass is then spread over `parts` blocks per row, and sample_kernel
+// starts from their results.
+__global__ __launch_bounds__(256) void sample_first_pass_kernel(SampleArgs a) {
+  __shared__ float red[32];
+  __shared__ int redi[32];
+  __shared__ float part[32];
+  const int r = blockIdx.x, p = blockIdx.y, V = a.vocab;
+  const RowOptions o = row_options(a, r);
+  const int chunk = (((V + a.parts - 1) / a.parts) + 3) & ~3;
+  const int lo = min(p * chunk, V), hi = min(lo + chunk, V);
+  float m = -INFINITY, ssum = 0.f;
+  int bi = 0x7fffffff;
+  first_pass(o, a.logits + (size_t)r * V, a.work + (size_t)r * V, lo, hi, V, m, ssum, bi);
+  block_merge(m, ssum, bi, red, part, redi);
+  if (threadIdx.x == 0) {
+    float* dst = a.partials + ((size_t)r * a.parts + p) * 4;
+    dst[0] = red[24];
+    dst[1] = red[25];
+    dst[2] = __int_as_float(redi[24]);
+  }
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
+  __shared__ float red[32];
+  __shared__ int redi[32];
+  __shared__ float part[SAMPLE_THREADS];
+  const int r = blockIdx.x, V = a.vocab, tid = threadIdx.x;
+  const float* lg = a.logits + (size_t)r * V;
+  float* x = a.work + (size_t)r * V;
+  const int sl = a.slot[r];
+  const float* fp = a.fparams + (size_t)sl * 8;
+  const float temp = fp[0], topp = fp[1], minp = fp[2];
+  const RowOptions o = row_options(a, r);
+  const bool greedy = o.greedy;
+  float m = -INFINITY, ssum = 0.f;
+  int bi = 0x7fffffff;
+  if (a.parts > 0) {  // the first pass has run; its parts are merged in order
+    if (tid < a.parts) {
+      const float* src = a.partials + ((size_t)r * a.parts + tid) * 4;
+      m = src[0]; ssum = src[1]; bi = __float_as_int(src[2]);
     }
-    __syncthreads();
+  } else {
+    first_pass(o, lg, x, 0, V, V, m, ssum, bi);
   }
+  block_merge(m, ssum, bi, red, part, redi);
+  if (tid == 0 && redi[24] == 0x7fffffff) redi[24] = 0;  // a row of NaNs
+  __syncthreads();
   const float mx = red[24];
   const int best = redi[24];
 
@@ -314,6 +369,12 @@ extern "C" int qrt_sample(const SampleArgs* args, hipStream_t stream) {
   SampleArgs a = *args;
   QRT_CHECK(a.rows >= 0 && a.vocab > 0, "sample: bad sizes");
   if (a.rows == 0) return 0;
+  QRT_CHECK(a.parts >= 0 && a.parts <= 64 && (a.parts == 0 || a.partials), "sample: bad number of parts %d", a.parts);
+  if (a.parts > 0) {
+    QRT_CHECK(a.rows <= 65535, "sample: %d rows in parts", a.rows);
+    sample_first_pass_kernel<<<dim3(a.rows, a.parts), dim3(256), 0, stream>>>(a);
+    QRT_LAUNCH_CHECK("sample (first pass)");
+  }
   sample_kernel<<<dim3(a.rows), dim3(SAMPLE_THREADS), 0, stream>>>(a);
   QRT_LAUNCH_CHECK("sample");
   return 0;

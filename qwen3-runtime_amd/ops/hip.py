@@ -72,7 +72,7 @@ class _SampleArgs(Structure):
         ("logits", c_void_p), ("work", c_void_p), ("counts", c_void_p), ("slot", c_void_p),
         ("fparams", c_void_p), ("iparams", c_void_p), ("seeds", c_void_p),
         ("out_token", c_void_p), ("out_logprob", c_void_p), ("rows", c_int), ("vocab", c_int),
-        ("write_work", c_int),
+        ("write_work", c_int), ("partials", c_void_p), ("parts", c_int),
     ]
 
 
@@ -516,6 +516,11 @@ class HipOps:
         a.fparams, a.iparams, a.seeds = fparams.data_ptr(), iparams.data_ptr(), seeds.data_ptr()
         a.out_token, a.out_logprob, a.rows, a.vocab = tok.data_ptr(), lp.data_ptr(), r, v
         a.write_work = 1 if keep_processed else 0  # greedy rows skip the write unless asked
+        # few rows: the first pass over each row is spread over blocks (about 256 in all)
+        parts = min(64, 256 // r, v // 2048) if r <= 64 else 0
+        if parts >= 2:
+            partials = torch.empty((r, parts, 4), dtype=torch.float32, device=logits.device)
+            a.partials, a.parts = partials.data_ptr(), parts
         self._check(self.lib, self.lib.qrt_sample(byref(a), _stream()))
         return tok, lp, work
 

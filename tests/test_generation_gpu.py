@@ -192,6 +192,38 @@ def test_sampler_filters_match_plain_and_draws_follow_the_distribution():
         torch.testing.assert_close(got_lp, want[tok_t].log(), atol=2e-3, rtol=2e-3)
 
 
+@pytest.mark.parametrize("v", [8192, 151936, 10001])
+def test_sampler_first_pass_in_parts_equals_one_block_per_row(v):
+    """Few rows and a large vocabulary: the first pass over a row runs in several blocks. Tokens,
+    log-probabilities and processed logits equal those of the one-block path (many rows), greedy
+    rows pick torch's first maximum, ties included."""
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    torch.manual_seed(3)
+    x = (torch.randn(5, v) * 2.0).to(DEV)
+    x[1, 77] = x[1, v - 5] = x[1].max() + 1.0          # a tie far apart: the lower id wins
+    seen = {i: [3, 3, 77, v - 1, 500] for i in range(5)}
+    params = [(SamplingParams(), 0), (SamplingParams(), 0),
+              (SamplingParams(temperature=0.8), 11),
+              (SamplingParams(temperature=1.2, top_k=40, top_p=0.9), 12),
+              (SamplingParams(temperature=0.0, repetition_penalty=1.5, presence_penalty=0.3, frequency_penalty=0.1), 0)]
+    reqs = [_Req(p) for p, _ in params]
+    s, rows = sample_rows(x, params, seen)
+    tok_parts, lp_parts = s.sample(x, rows, reqs)
+    # the one-block path: the same five rows among many (parts are used up to 64 rows)
+    many = x.repeat(14, 1).contiguous()
+    params_many = params * 14
+    s2, rows2 = sample_rows(many, params_many, {i: seen[0] for i in range(70)})
+    tok_one, lp_one = s2.sample(many, rows2, [_Req(p) for p, _ in params_many])
+    if v >= 4096:
+        assert min(64, 256 // 5, v // 2048) >= 2       # the first call did run in parts
+    assert tok_parts == tok_one[:5]
+    torch.testing.assert_close(torch.tensor(lp_parts), torch.tensor(lp_one[:5]), atol=1e-5, rtol=1e-5)
+    assert tok_parts[0] == int(torch.argmax(x[0]))
+    assert tok_parts[1] == 77
+    assert lp_parts[0] == pytest.approx(float(torch.log_softmax(x[0].double(), -1).max()), abs=1e-4)
+
+
 def test_sampler_is_seeded_and_counter_based():
     from qwen3_runtime_amd.sampling.params import SamplingParams
 
