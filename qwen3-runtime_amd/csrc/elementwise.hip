@@ -39,8 +39,11 @@ extern "C" int qrt_embed(const int* ids, const void* table, int table_dtype, flo
 // (rows up to 256 * VEC * KEEP wide; wider rows are read a second time), all loads of a row are
 // issued before the first use, squares are summed over the block in a fixed order.
 // delta may come as `planes` planes [planes, T, H] that are added in order (the parts of a product
-// whose K was cut).
-template <typename TD, typename TO, int VEC, int KEEP>
+// whose K was cut). PL is the number of planes where it is known when compiling (0: no delta):
+// residual, planes and weights are then all loaded at once, unconditionally (clamped index), so
+// that a row costs one round of memory latency instead of one per plane and one for the weights;
+// PL = -1 loops over any number of planes.
+template <typename TD, typename TO, int VEC, int KEEP, int PL>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                                           const float* __restrict__ weight,
                                                           const int* __restrict__ rows, TO* __restrict__ out,
@@ -57,22 +60,37 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ re
   constexpr int STRIDE = 256 * VEC;
   const int i0 = threadIdx.x * VEC;
 
-  fvec_t x[KEEP];
+  fvec_t x[KEEP], w[KEEP];
   float ss = 0.f;
+  if (PL >= 0) {
+    dvec_t d[PL > 0 ? PL : 1][KEEP];
 #pragma unroll
-  for (int j = 0; j < KEEP; ++j) {
-    const int i = i0 + j * STRIDE;
+    for (int j = 0; j < KEEP; ++j) {
+      const int ic = min(i0 + j * STRIDE, hidden - VEC);  // beyond the row: some element of it, dropped below
+      x[j] = *(const fvec_t*)(res + ic);
+      w[j] = *(const fvec_t*)(weight + ic);
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) x[j][e] = 0.f;
-    if (i < hidden) x[j] = *(const fvec_t*)(res + i);
-  }
-  if (del) {
-    for (int p = 0; p < planes; ++p) {
+      for (int p = 0; p < PL; ++p) d[p][j] = *(const dvec_t*)(del + p * plane_stride + ic);
+    }
 #pragma unroll
-      for (int j = 0; j < KEEP; ++j) {
-        const int i = i0 + j * STRIDE;
-        if (i < hidden) {
-          const dvec_t d = *(const dvec_t*)(del + p * plane_stride + i);
+    for (int p = 0; p < PL; ++p)
+#pragma unroll
+      for (int j = 0; j < KEEP; ++j)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[j][e] += to_f32<TD>(d[p][j][e]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < KEEP; ++j) {
+      const int ic = min(i0 + j * STRIDE, hidden - VEC);
+      x[j] = *(const fvec_t*)(res + ic);
+      w[j] = *(const fvec_t*)(weight + ic);
+    }
+    if (del) {
+      for (int p = 0; p < planes; ++p) {
+#pragma unroll
+        for (int j = 0; j < KEEP; ++j) {
+          const int ic = min(i0 + j * STRIDE, hidden - VEC);
+          const dvec_t d = *(const dvec_t*)(del + p * plane_stride + ic);
 #pragma unroll
           for (int e = 0; e < VEC; ++e) x[j][e] += to_f32<TD>(d[e]);
         }
@@ -108,10 +126,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ re
   for (int j = 0; j < KEEP; ++j) {
     const int i = i0 + j * STRIDE;
     if (i < hidden) {
-      const fvec_t w = *(const fvec_t*)(weight + i);
       ovec_t y;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) y[e] = from_f32<TO>(x[j][e] * inv * w[e]);
+      for (int e = 0; e < VEC; ++e) y[e] = from_f32<TO>(x[j][e] * inv * w[j][e]);
       *(ovec_t*)(o + i) = y;
     }
   }
@@ -124,10 +141,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ re
         for (int e = 0; e < VEC; ++e) v[e] += to_f32<TD>(d[e]);
       }
     }
-    const fvec_t w = *(const fvec_t*)(weight + i);
+    const fvec_t wv = *(const fvec_t*)(weight + i);
     ovec_t y;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) y[e] = from_f32<TO>(v[e] * inv * w[e]);
+    for (int e = 0; e < VEC; ++e) y[e] = from_f32<TO>(v[e] * inv * wv[e]);
     *(ovec_t*)(o + i) = y;
   }
 }
@@ -141,16 +158,20 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
   dim3 grid(num_out_rows), block(256);
   const bool vec4 = hidden % 4 == 0 && (uintptr_t)residual % 16 == 0 && (uintptr_t)weight % 16 == 0 &&
                     (uintptr_t)out % 16 == 0 && (!delta || (uintptr_t)delta % 16 == 0) && plane_stride % 4 == 0;
+  // planes known to the compiler (0: no delta) where the count is a usual one
+  const int pl = !delta ? 0 : (planes == 1 || planes == 2 || planes == 4) ? planes : -1;
+#define GO(TD, TO, VEC, KEEP, PL)                                                                               \
+  add_rmsnorm_kernel<TD, TO, VEC, KEEP, PL><<<grid, block, 0, stream>>>(residual, (const TD*)delta, weight,     \
+                                                                        rows, (TO*)out, hidden, eps, planes,    \
+                                                                        (size_t)plane_stride)
 #define LAUNCH(TD, TO)                                                                                          \
   do {                                                                                                          \
-    if (vec4)                                                                                                   \
-      add_rmsnorm_kernel<TD, TO, 4, 4><<<grid, block, 0, stream>>>(residual, (const TD*)delta, weight, rows,    \
-                                                                   (TO*)out, hidden, eps, planes,               \
-                                                                   (size_t)plane_stride);                       \
-    else                                                                                                        \
-      add_rmsnorm_kernel<TD, TO, 1, 8><<<grid, block, 0, stream>>>(residual, (const TD*)delta, weight, rows,    \
-                                                                   (TO*)out, hidden, eps, planes,               \
-                                                                   (size_t)plane_stride);                       \
+    if (!vec4) GO(TD, TO, 1, 8, -1);                                                                            \
+    else if (pl == 0) GO(TD, TO, 4, 4, 0);                                                                      \
+    else if (pl == 1) GO(TD, TO, 4, 4, 1);                                                                      \
+    else if (pl == 2) GO(TD, TO, 4, 4, 2);                                                                      \
+    else if (pl == 4) GO(TD, TO, 4, 4, 4);                                                                      \
+    else GO(TD, TO, 4, 4, -1);                                                                                  \
   } while (0)
   if (delta_dtype == QRT_F32 && out_dtype == QRT_F32) LAUNCH(float, float);
   else if (delta_dtype == QRT_BF16 && out_dtype == QRT_BF16) LAUNCH(bf16_t, bf16_t);
@@ -158,6 +179,7 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
   else if (delta_dtype == QRT_BF16 && out_dtype == QRT_F32) LAUNCH(bf16_t, float);
   else return qrt_fail("add_rmsnorm: unknown dtypes %d %d", delta_dtype, out_dtype);
 #undef LAUNCH
+#undef GO
   QRT_LAUNCH_CHECK("add_rmsnorm");
   return 0;
 }

@@ -60,6 +60,29 @@ def test_add_rmsnorm(ops, dtype, t, h, eps):
     close(ops.add_rmsnorm(res.clone(), None, w, eps, dtype), R.add_rmsnorm(res.clone(), None, w, eps, dtype), tol, tol)
 
 
+@pytest.mark.parametrize("planes", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("t,h", [(3, 2560), (2, 5000), (4, 4096), (5, 101), (1, 8)])
+def test_add_rmsnorm_sums_planes_in_order(ops, planes, t, h):
+    """The delta in planes [P, T, H] (float32): the residual becomes ((res + p0) + p1) + ..., bit
+    for bit, for plane counts the kernel unrolls (1, 2, 4) and those it loops over, for rows held
+    in registers, rows wider than that (5,000) and rows that cannot be read four at a time (101)."""
+    res = rnd(t, h, seed=1)
+    delta = rnd(planes, t, h, seed=2)
+    w = (1 + 0.1 * rnd(h, seed=3)).contiguous()
+    want_res = res.clone()
+    for p in range(planes):
+        want_res = want_res + delta[p]
+    got_res = res.clone()
+    got = ops.add_rmsnorm(got_res, delta, w, 1e-6, torch.bfloat16)
+    close(got_res, want_res, 0, 0)
+    close(got, R.add_rmsnorm(want_res.clone(), None, w, 1e-6, torch.bfloat16), 1e-2, 1e-2)
+    rows = torch.tensor([t - 1, 0], dtype=torch.int32, device=DEV)
+    untouched = res.clone()
+    sel = ops.add_rmsnorm(untouched, delta, w, 1e-6, torch.bfloat16, rows)
+    close(untouched, res, 0, 0)
+    close(sel, got[rows.long()], 0, 0)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu(ops, dtype):
     gu = rnd(11, 2 * 272, dtype=dtype, scale=3.0)
