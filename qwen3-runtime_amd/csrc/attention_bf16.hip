@@ -596,7 +596,9 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int seq = a.tile_seq[blockIdx.x];
+  // every sequence is one tile here, so the tile list is not read: one dependent load less
+  // before the first key arrives
+  const int seq = blockIdx.x;
   const int kvh = blockIdx.y, split = blockIdx.z;
   const int g = a.nq / a.nkv;
   const int q_begin = a.cu_q[seq];
@@ -695,7 +697,8 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
   }
 }
 
-// tiles must all have at most 16 rows (max_q_len * g <= 16) and D <= 256
+// every sequence at most 16 rows (max_q_len * g <= 16) and D <= 256; num_tiles = number of
+// sequences, the tile lists are not read
 extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_total, hipStream_t stream) {
   AttnTileArgs a = *args;
   QRT_CHECK(a.nq > 0 && a.nkv > 0 && a.nq % a.nkv == 0, "attention: %d query heads do not divide into %d key heads",

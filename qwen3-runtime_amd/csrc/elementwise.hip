@@ -292,42 +292,50 @@ __global__ void qk_norm_rope_store_kernel(QkArgs a) {
                       : (const T*)a.k_in + (size_t)t * a.k_stride + (size_t)hh * D;
   const float* w = is_q ? a.q_weight : a.k_weight;
 
-  // each lane owns the pairs (p, p + D/2) for p = lane, lane + 64, ... (D <= 512)
-  float x1[4], x2[4];
+  // each lane owns the pairs (p, p + D/2) for p = lane, lane + 64, ... (D <= 512).
+  // Everything the lane will need is loaded before the first use (norm weights, position,
+  // frequencies, slot), so that the kernel costs one round of memory latency, not four.
+  float x1[4], x2[4], w1[4], w2[4], fr[4];
   float ss = 0.f;
+  const float pos = a.inv_freq ? (float)a.positions[t] : 0.f;
+  const int slot = (!is_q && a.slots) ? a.slots[t] : 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int p = lane + 64 * i;
     x1[i] = x2[i] = 0.f;
+    w1[i] = w2[i] = 1.f;
+    fr[i] = 0.f;
     if (p < half) {
       x1[i] = to_f32<T>(src[p]);
       x2[i] = to_f32<T>(src[p + half]);
-      ss += x1[i] * x1[i] + x2[i] * x2[i];
+      if (w) {
+        w1[i] = w[p];
+        w2[i] = w[p + half];
+      }
+      if (a.inv_freq) fr[i] = a.inv_freq[p];
     }
   }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) ss += x1[i] * x1[i] + x2[i] * x2[i];
   if (w) {
     ss = wave_sum(ss);
     const float inv = rsqrtf(ss / (float)D + a.eps);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int p = lane + 64 * i;
-      if (p < half) {
-        x1[i] = x1[i] * inv * w[p];
-        x2[i] = x2[i] * inv * w[p + half];
-      }
+      x1[i] = x1[i] * inv * w1[i];
+      x2[i] = x2[i] * inv * w2[i];
     }
   }
   if (a.inv_freq) {
-    const float pos = (float)a.positions[t];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int p = lane + 64 * i;
       if (p < half) {
-        const float ang = pos * a.inv_freq[p];
-        float s, c;
-        sincosf(ang, &s, &c);
-        const float y1 = x1[i] * c - x2[i] * s;
-        const float y2 = x2[i] * c + x1[i] * s;
+        const float ang = pos * fr[i];
+        float sn, c;
+        sincosf(ang, &sn, &c);
+        const float y1 = x1[i] * c - x2[i] * sn;
+        const float y2 = x2[i] * c + x1[i] * sn;
         x1[i] = y1;
         x2[i] = y2;
       }
@@ -338,7 +346,6 @@ __global__ void qk_norm_rope_store_kernel(QkArgs a) {
   if (!is_q && a.k_out) dense = (T*)a.k_out + ((size_t)t * a.nkv + hh) * D;
   T* paged = nullptr;
   if (!is_q && a.slots) {
-    const int slot = a.slots[t];
     const int page = slot / a.page_size, off = slot - page * a.page_size;
     paged = (T*)a.k_cache + (((size_t)page * a.nkv + hh) * a.page_size + off) * D;
   }

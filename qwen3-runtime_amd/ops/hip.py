@@ -455,14 +455,17 @@ class HipOps:
         waves = 1 if max_rows <= 16 else (2 if max_rows <= 32 else 4)
         # long portions: several row tiles per wave, so that loaded keys and values serve more rows
         row_tiles = 1 if max_rows <= 64 else (self.prefill_row_tiles if d <= 128 else min(2, self.prefill_row_tiles))
-        key = ("attn_tiles", g, waves, row_tiles)
-        plan = ctx.scratch.get(key)
-        if plan is None:
-            host, n_tiles = self.plan_tiles(ctx.q_lens_host, ctx.kv_lens_host, g, 16 * waves * row_tiles, nkv,
-                                            self.resident_blocks if waves == 4 and row_tiles >= 2 else 0)
-            plan = (torch.from_numpy(host).to(q.device), n_tiles)
-            ctx.scratch[key] = plan
-        tiles, n_tiles = plan
+        if decode:
+            tiles, n_tiles = None, ctx.num_seqs  # every sequence is one tile; the kernel needs no list
+        else:
+            key = ("attn_tiles", g, waves, row_tiles)
+            plan = ctx.scratch.get(key)
+            if plan is None:
+                host, n_tiles = self.plan_tiles(ctx.q_lens_host, ctx.kv_lens_host, g, 16 * waves * row_tiles, nkv,
+                                                self.resident_blocks if waves == 4 and row_tiles >= 2 else 0)
+                plan = (torch.from_numpy(host).to(q.device), n_tiles)
+                ctx.scratch[key] = plan
+            tiles, n_tiles = plan
         splits = ctx.scratch.get("attn_splits") or (
             self.choose_decode_splits(n_tiles, nkv, ctx.max_kv_len) if decode
             else self.choose_splits(n_tiles, nkv, ctx.max_kv_len))
@@ -471,8 +474,9 @@ class HipOps:
         a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
         a.kv_lens = _need(ctx.kv_lens, "kv_lens", torch.int32, (ctx.num_seqs,)).data_ptr()
         a.block_table, a.table_width = cache.group.block_table.data_ptr(), cache.group.block_table.shape[1]
-        a.tile_seq = tiles.data_ptr()
-        a.tile_row0 = tiles.data_ptr() + 4 * n_tiles
+        if tiles is not None:
+            a.tile_seq = tiles.data_ptr()
+            a.tile_row0 = tiles.data_ptr() + 4 * n_tiles
         a.num_tiles, a.nq, a.nkv, a.page_size, a.window = n_tiles, nq, nkv, cache.group.page_size, window
         a.num_splits, a.waves, a.row_tiles = splits, waves, row_tiles
         a.use_lds = 1 if self.prefill_through_lds else 0
