@@ -20,8 +20,8 @@
 // which stores values transposed ([page, head, D, offset]). No data crosses
 // lanes except the row maximum and sum.
 //
-// Softmax is online, float32, in base 2 (scores pre-multiplied by
-// scale * log2 e); probabilities are rounded to bfloat16 for the second
+// Softmax is online, float32, in base 2 (scale * log2 e is folded into the
+// exponent's argument); probabilities are rounded to bfloat16 for the second
 // product, accumulation is float32. Key j is visible to the row at position p
 // iff j <= p and (no window or j > p - window).
 #include "common.h"
