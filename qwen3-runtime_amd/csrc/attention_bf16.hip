@@ -294,7 +294,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   extern __shared__ bf16_t lds_kv[];  // [2][STAGE_ELEMS]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int tile = blockIdx.x / a.nkv, kvh = blockIdx.x - tile * a.nkv;
+  const int tile = blockIdx.x / a.nkv, kvh = blockIdx.x - tile * a.nkv, split = blockIdx.z;
   const int seq = a.tile_seq[tile];
   const int g = a.nq / a.nkv;
   const int q_begin = a.cu_q[seq];
@@ -335,7 +335,10 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   const int blk_last_row = min(tile_row0 + 64 * RT - 1, n_rows - 1);
   const int blk_pos_min = first_pos + tile_row0 / g, blk_pos_max = first_pos + blk_last_row / g;
   const int lo = a.window > 0 ? max(0, blk_pos_min - a.window + 1) : 0;
-  const int b0 = lo >> 5, b1 = (blk_pos_max >> 5) + 1;
+  // the blocks of keys of this block of waves, and of them the part of this split
+  const int all_b0 = lo >> 5, all_b1 = (blk_pos_max >> 5) + 1;
+  const int per = (all_b1 - all_b0 + a.num_splits - 1) / a.num_splits;
+  const int b0 = all_b0 + split * per, b1 = min(all_b1, b0 + per);
   int wb0 = b1, wb1 = b0;  // this wave's blocks: none unless it has rows
   if (wave_has_rows) {
     const int row_last = min(row0 + 16 * RT - 1, n_rows - 1);
@@ -418,10 +421,12 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   };
 
   int kpage[PIECES], vpage[PIECES];
-  lookup(b0, kpage, vpage);
-  fetch(b0, kpage, vpage);
-  if (b0 + 1 < b1) lookup(b0 + 1, kpage, vpage);
-  stash(b0, 0);
+  if (b0 < b1) {  // a split may be left without blocks
+    lookup(b0, kpage, vpage);
+    fetch(b0, kpage, vpage);
+    if (b0 + 1 < b1) lookup(b0 + 1, kpage, vpage);
+    stash(b0, 0);
+  }
   __syncthreads();
   for (int b = b0; b < b1; ++b) {
     const int stage = (b - b0) & 1;
@@ -471,15 +476,25 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
     float lt = l[t];
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
-    if (!row_valid[t]) continue;
+    if (!row_valid[t] || !wave_has_rows) continue;
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
-    bf16_t* op = a.out + row_index[t] * D;
+    if (a.num_splits == 1) {
+      bf16_t* op = a.out + row_index[t] * D;
 #pragma unroll
-    for (int i = 0; i < DB; ++i) {
-      bf16x4_t w;
+      for (int i = 0; i < DB; ++i) {
+        bf16x4_t w;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) w[r] = (bf16_t)(o[t][i][r] * inv);
-      *(bf16x4_t*)(op + 16 * i + 4 * quad) = w;
+        for (int r = 0; r < 4; ++r) w[r] = (bf16_t)(o[t][i][r] * inv);
+        *(bf16x4_t*)(op + 16 * i + 4 * quad) = w;
+      }
+    } else {
+      float* op = a.part_o + (row_index[t] * a.num_splits + split) * D;
+#pragma unroll
+      for (int i = 0; i < DB; ++i) {
+        f32x4_t w = o[t][i] * inv;
+        *(f32x4_t*)(op + 16 * i + 4 * quad) = w;
+      }
+      if (quad == 0) a.part_lse[row_index[t] * a.num_splits + split] = lt > 0.f ? m[t] + log2f(lt) : -INFINITY;
     }
   }
 }
@@ -740,15 +755,12 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
   QRT_CHECK((long long)a.num_tiles * a.nkv < (1ll << 31), "attention: %d tiles x %d key heads is too many blocks", a.num_tiles, a.nkv);
   dim3 grid(a.num_tiles * a.nkv, 1, a.num_splits), block(64 * a.waves);
-  if (a.row_tiles == 2 && a.waves == 4 && a.num_splits == 1 && a.use_lds) {
+  if (a.row_tiles == 2 && a.waves == 4 && a.use_lds) {
     const size_t smem = 2 * (size_t)STAGE_ELEMS * sizeof(bf16_t);
     QRT_CHECK(smem <= 64 * 1024, "attention: head size %d needs %zu bytes of LDS", D, smem);
     if (p2) attention_bf16_prefill_kernel<2, true><<<grid, block, smem, stream>>>(a);
     else attention_bf16_prefill_kernel<2, false><<<grid, block, smem, stream>>>(a);
-    QRT_LAUNCH_CHECK("attention_bf16_prefill");
-    return 0;
-  }
-  if (a.row_tiles == 1 && p2) attention_bf16_kernel<1, true><<<grid, block, 0, stream>>>(a);
+  } else if (a.row_tiles == 1 && p2) attention_bf16_kernel<1, true><<<grid, block, 0, stream>>>(a);
   else if (a.row_tiles == 1) attention_bf16_kernel<1, false><<<grid, block, 0, stream>>>(a);
   else if (a.row_tiles == 2 && p2) attention_bf16_kernel<2, true><<<grid, block, 0, stream>>>(a);
   else if (a.row_tiles == 2) attention_bf16_kernel<2, false><<<grid, block, 0, stream>>>(a);

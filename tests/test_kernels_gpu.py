@@ -397,6 +397,22 @@ def test_paged_attention_splits_agree(ops):
         close(got, want, 2e-2, 2e-2)
 
 
+@pytest.mark.parametrize("seqs,nq,nkv,d,ps,window", [([(100, 1500), (30, 30)], 8, 2, 64, 16, None),
+                                                     ([(300, 700)], 4, 1, 128, 8, None),
+                                                     ([(90, 1200), (70, 75)], 6, 2, 32, 24, 200)])
+def test_long_portions_split_over_blocks_agree(ops, seqs, nq, nkv, d, ps, window):
+    """Portions of more than 64 rows (the kernel that shares keys through LDS) with the keys cut
+    over 1 to 40 blocks: splits without a block of keys, a window, a page size that is no power
+    of two."""
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, window=window)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, 0.125, window)
+    for splits in (1, 2, 3, 40):
+        ctx.scratch["attn_splits"] = splits
+        got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 0.125, window)
+        close(got, want, 2e-2, 2e-2)
+
+
 def test_decode_attention_many_sequences_and_repeated_launches(ops):
     """Many sequences of very different lengths, launched again and again with other split counts."""
     g = torch.Generator().manual_seed(5)
