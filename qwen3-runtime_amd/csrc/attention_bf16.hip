@@ -135,6 +135,48 @@ __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t*
   for (int i = 0; i < DB; ++i) o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[i], pb, o[i], 0, 0, 0);
 }
 
+// ------------------------------------------------ keys and values straight from the pages
+struct KvBlock {  // the keys and values of one block of 32 keys, as MFMA operands
+  bf16x8_t k[2][KFULL > 0 ? KFULL : 1];
+  bf16x8_t kt[2];
+  bf16x8_t v[DB];
+};
+
+// Every load is unconditional: positions are clamped into [lo, pos_max], which lies in pages
+// the sequence holds; what was read from a clamped place is masked (keys) or zeroed (values)
+// before use. Loads under branches would make the compiler wait for all loads in flight
+// wherever it can no longer count them.
+template <bool P2>
+__device__ __forceinline__ void block_pages(const int* __restrict__ table, int base, int lo, int pos_max, int ps,
+                                            int r16, int quad, int pg[3]) {
+  const int psh = __builtin_ctz(ps);
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
+    pg[kb] = table[page_div<P2>(kidx, ps, psh)];
+  }
+  const int kv0 = min(max(base + 8 * quad, lo & ~7), pos_max & ~7);
+  pg[2] = table[page_div<P2>(kv0, ps, psh)];
+}
+
+template <bool P2>
+__device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int base, int lo, int pos_max, int r16,
+                                           int quad, const int pg[3], KvBlock& blk) {
+  const int ps = a.page_size;
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) {
+    const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
+    const bf16_t* kp = a.k_cache + (((size_t)pg[kb] * a.nkv + kvh) * ps + page_mod<P2>(kidx, ps)) * D;
+#pragma unroll
+    for (int i = 0; i < KFULL; ++i) blk.k[kb][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
+    if (KTAIL) blk.kt[kb] = load_tail(kp + 32 * KFULL, quad);
+  }
+  const int kv0 = min(max(base + 8 * quad, lo & ~7), pos_max & ~7);
+  const bf16_t* vp = a.v_cache + (((size_t)pg[2] * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps);
+#pragma unroll
+  for (int i = 0; i < DB; ++i) blk.v[i] = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
+}
+
 // General kernel (prompt portions and mixed batches). A wave owns RT tiles of 16
 // rows each, 16 * RT consecutive rows of the sequence's row matrix; a block is
 // four waves, 64 * RT rows. The keys and values of a block of 32 keys are read
@@ -202,50 +244,43 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
     for (int i = 0; i < DB; ++i) o[t][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int b = b0; b < b1; ++b) {
-    const int base = b << 5;
-    // keys of the block as A operands: row 4 quad' + r of sub-block kb holds key 8 quad' + 4 kb + r
-    bf16x8_t kk[2][KFULL > 0 ? KFULL : 1], kt[2];
+  // page numbers are looked up one block ahead of the loads that need them; all loads are
+  // unconditional (clamped), see block_pages / block_load
+  if (b0 < b1) {
+    int pg[3], pg_next[3];
+    block_pages<P2>(table, b0 << 5, lo, pos_max, ps, r16, quad, pg);
+    for (int b = b0; b < b1; ++b) {
+      const int base = b << 5;
+      KvBlock blk;
+      block_load<P2>(a, kvh, base, lo, pos_max, r16, quad, pg, blk);
+      block_pages<P2>(table, min(b + 1, b1 - 1) << 5, lo, pos_max, ps, r16, quad, pg_next);
+      // values of keys outside [lo, pos_max] came from a clamped place and may be anything
+      const int kv0 = base + 8 * quad;
+      if (base < lo || base + 31 > pos_max) {  // the same for the whole wave
+        const bool seen = kv0 <= pos_max && kv0 + 7 >= lo;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      int kidx = base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3);
-      kidx = min(max(kidx, lo), pos_max);  // stay inside pages this sequence holds; masked below
-      const int page = table[page_div<P2>(kidx, ps, psh)];
-      const bf16_t* kp = a.k_cache + (((size_t)page * a.nkv + kvh) * ps + page_mod<P2>(kidx, ps)) * D;
+        for (int i = 0; i < DB; ++i)
 #pragma unroll
-      for (int i = 0; i < KFULL; ++i) kk[kb][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
-      if (KTAIL) kt[kb] = load_tail(kp + 32 * KFULL, quad);
-    }
-    // values: 8 consecutive keys base + 8 quad .. + 7 of head element 16 i + r16
-    const int kv0 = base + 8 * quad;
-    const bool vload = kv0 <= pos_max && kv0 + 7 >= lo;
-    const int vpage = vload ? table[page_div<P2>(kv0, ps, psh)] : 0;
-    const bf16_t* vp = a.v_cache + (((size_t)vpage * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps);
-    bf16x8_t vv[DB];
-#pragma unroll
-    for (int i = 0; i < DB; ++i) {
-      if (vload) vv[i] = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
-      else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) vv[i][e] = (bf16_t)0.0f;
+          for (int e = 0; e < 8; ++e) blk.v[i][e] = seen ? blk.v[i][e] : (bf16_t)0.0f;
       }
-    }
-
 #pragma unroll
-    for (int t = 0; t < RT; ++t) {
-      f32x4_t s[2];
+      for (int t = 0; t < RT; ++t) {
+        f32x4_t s[2];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        for (int kb = 0; kb < 2; ++kb) {
+          f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < KFULL; ++i)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk[kb][i], qreg[t][i], acc, 0, 0, 0);
-        if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[kb], qtail[t], acc, 0, 0, 0);
-        s[kb] = acc;
+          for (int i = 0; i < KFULL; ++i)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[kb][i], qreg[t][i], acc, 0, 0, 0);
+          if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kt[kb], qtail[t], acc, 0, 0, 0);
+          s[kb] = acc;
+        }
+        // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
+        const bool whole = base + 31 <= tile_pos_min[t] && (a.window == 0 || base > tile_pos_max[t] - a.window);
+        tile_update(s, blk.v, !whole, base, quad, row_valid[t], qpos[t], a.window, a.scale_log2, m[t], l[t], o[t]);
       }
-      // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
-      const bool whole = base + 31 <= tile_pos_min[t] && (a.window == 0 || base > tile_pos_max[t] - a.window);
-      tile_update(s, vv, !whole, base, quad, row_valid[t], qpos[t], a.window, a.scale_log2, m[t], l[t], o[t]);
+#pragma unroll
+      for (int i = 0; i < 3; ++i) pg[i] = pg_next[i];
     }
   }
 
@@ -533,47 +568,6 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
 // needs a device-scope fence in every block; with one L2 per XCD that fence costs
 // more than the second launch: measured 355 us against 98 us at 64 sequences.)
 constexpr int DW = 4;
-
-struct KvBlock {  // the keys and values of one block of 32 keys, as MFMA operands
-  bf16x8_t k[2][KFULL > 0 ? KFULL : 1];
-  bf16x8_t kt[2];
-  bf16x8_t v[DB];
-};
-
-// Every load is unconditional: positions are clamped into [lo, pos_max], which lies in pages
-// the sequence holds; what was read from a clamped place is masked (keys) or zeroed (values)
-// before use. Loads under branches would make the compiler wait for all loads in flight
-// wherever it can no longer count them.
-template <bool P2>
-__device__ __forceinline__ void block_pages(const int* __restrict__ table, int base, int lo, int pos_max, int ps,
-                                            int r16, int quad, int pg[3]) {
-  const int psh = __builtin_ctz(ps);
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb) {
-    const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
-    pg[kb] = table[page_div<P2>(kidx, ps, psh)];
-  }
-  const int kv0 = min(max(base + 8 * quad, lo & ~7), pos_max & ~7);
-  pg[2] = table[page_div<P2>(kv0, ps, psh)];
-}
-
-template <bool P2>
-__device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int base, int lo, int pos_max, int r16,
-                                           int quad, const int pg[3], KvBlock& blk) {
-  const int ps = a.page_size;
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb) {
-    const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
-    const bf16_t* kp = a.k_cache + (((size_t)pg[kb] * a.nkv + kvh) * ps + page_mod<P2>(kidx, ps)) * D;
-#pragma unroll
-    for (int i = 0; i < KFULL; ++i) blk.k[kb][i] = *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
-    if (KTAIL) blk.kt[kb] = load_tail(kp + 32 * KFULL, quad);
-  }
-  const int kv0 = min(max(base + 8 * quad, lo & ~7), pos_max & ~7);
-  const bf16_t* vp = a.v_cache + (((size_t)pg[2] * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps);
-#pragma unroll
-  for (int i = 0; i < DB; ++i) blk.v[i] = *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
-}
 
 __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg, bf16x8_t qtail, int base, int lo,
                                               int pos_min, int pos_max, int quad, bool row_valid, int qpos,
