@@ -61,6 +61,38 @@ def test_graph_replay_equals_eager(model_folders, dtype):
     assert m.generate(prompts, max_tokens=40) == eager
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_across_a_context_bucket(model_folders, dtype):
+    """A request that grows past 512 tokens while decoding moves to the graph of the next bucket
+    (wider block table, other key splits); a request that ends changes the batch size. The graphs
+    are fed the tokens of eager steps and must give them the log-probabilities eager steps gave
+    (a graph cuts the keys for its bucket's length, so bfloat16 differs by rounding); in float32
+    the tokens chosen freely are the same."""
+    cfg, _ = P.read_model(model_folders["tiny_b"])
+    prompts = prompts_for(cfg, [490, 20, 300], seed=5)
+    n_out = (60, 25, 60)
+
+    def run(graph, forced=None):
+        m = llm(model_folders["tiny_b"], dtype=dtype, pages=160, budget=128, graph=graph)
+        eng = m.engine
+        reqs = [eng.request(eng.add_request(p, n, forced_tokens=None if forced is None else forced[i]))
+                for i, (p, n) in enumerate(zip(prompts, n_out))]
+        while not eng.is_finished():
+            eng.step()
+        return m, [r.output_tokens for r in reqs], [r.logprobs for r in reqs]
+
+    _, want, want_lp = run(False)
+    m, got, got_lp = run(True, forced=want)
+    assert got == want
+    tol = 1e-4 if dtype == "float32" else 5e-2
+    for a, b in zip(got_lp, want_lp):
+        torch.testing.assert_close(torch.tensor(a), torch.tensor(b), atol=tol, rtol=tol)
+    keys = set(m.engine.runner._graphs)
+    assert {bucket for _, bucket in keys} >= {512, 1024} and {batch for batch, _ in keys} >= {2, 3}
+    if dtype == "float32":
+        assert run(True)[1] == want
+
+
 def test_preemption_does_not_change_tokens(model_folders):
     """12 pages of 8 for three requests that need 9 each: some are preempted and recomputed
     (reference: tests/invariance/test_preempt.py:10-33)."""
