@@ -106,6 +106,38 @@ def test_preemption_does_not_change_tokens(model_folders):
     assert m.engine.cache.num_free_pages == 12 and m.engine.cache.slots.num_free == 3
 
 
+@pytest.mark.parametrize("seed,graph", [(0, False), (1, True), (2, False)])
+def test_random_traffic_with_few_pages(model_folders, seed, graph):
+    """Requests of random lengths arriving at random steps into a pool too small for them:
+    portions, decoding, waiting, preemption and recomputation in every order the seed gives.
+    Every request ends with the tokens it gets when it runs alone; after every step no page is
+    lost or held twice, and at the end all pages and slots are free."""
+    import random
+
+    rng = random.Random(seed)
+    cfg, _ = P.read_model(model_folders["tiny_b"])
+    n = 14
+    prompts = prompts_for(cfg, [rng.randint(1, 90) for _ in range(n)], seed=seed)
+    n_out = [rng.randint(1, 20) for _ in range(n)]
+    arrive = sorted(rng.randint(0, 60) for _ in range(n))
+    alone = llm(model_folders["tiny_b"], pages=64, graph=False).engine
+    want = [alone.generate(p, max_tokens=k) for p, k in zip(prompts, n_out)]
+    m = llm(model_folders["tiny_b"], page=8, pages=17, seqs=4, budget=rng.choice([16, 40, 64]), graph=graph)
+    eng = m.engine
+    reqs, step = {}, 0
+    while len(reqs) < n or not eng.is_finished():
+        while len(reqs) < n and arrive[len(reqs)] <= step:
+            i = len(reqs)
+            reqs[i] = eng.request(eng.add_request(prompts[i], n_out[i]))
+        eng.step()
+        eng.cache.check()
+        step += 1
+        assert step < 5000, "the engine makes no progress"
+    assert [reqs[i].output_tokens for i in range(n)] == want
+    assert eng.scheduler.num_preemptions >= 1
+    assert eng.cache.num_free_pages == 17 and eng.cache.slots.num_free == 4
+
+
 def test_requests_arriving_mid_decode_and_seeded_sampling(model_folders):
     """Temperature 0.8 with per-request seeds: tokens do not depend on batch mates or admission time."""
     from qwen3_runtime_amd.sampling.params import SamplingParams
