@@ -41,6 +41,17 @@ template <typename T> __device__ __forceinline__ T from_f32(float x);
 template <> __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) { return (bf16_t)x; }
 
+// Sine and cosine of a rotation angle held in float32 (position times frequency: up to
+// millions of radians). The library routine reduces such arguments with a table it loads from
+// memory; here the angle is reduced to [-pi, pi] in float64 (exact to 1e-10 rad) first, so the
+// routine stays on its short path and the kernel has no loads in its middle. The result is the
+// sine and cosine of the float32 angle to within one unit in the last place.
+__device__ __forceinline__ void sincos_angle(float angle, float* sn, float* cs) {
+  const double turns = (double)angle * 0.15915494309189535;  // 1 / (2 pi)
+  const float reduced = (float)((turns - rint(turns)) * 6.283185307179586);
+  sincosf(reduced, sn, cs);
+}
+
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);

@@ -333,7 +333,7 @@ __global__ void qk_norm_rope_store_kernel(QkArgs a) {
       if (p < half) {
         const float ang = pos * fr[i];
         float sn, c;
-        sincosf(ang, &sn, &c);
+        sincos_angle(ang, &sn, &c);
         const float y1 = x1[i] * c - x2[i] * sn;
         const float y2 = x2[i] * c + x1[i] * sn;
         x1[i] = y1;
@@ -389,7 +389,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_wide_kernel(QkArgs a, 
     if (a.inv_freq) {
       const float pos = (float)a.positions[t];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) sincosf(pos * a.inv_freq[8 * c + e], &sn[e], &cs[e]);
+      for (int e = 0; e < 8; ++e) sincos_angle(pos * a.inv_freq[8 * c + e], &sn[e], &cs[e]);
     }
     const int slot = a.slots ? a.slots[t] : 0;
     const int page = slot / a.page_size, off = slot - page * a.page_size;
