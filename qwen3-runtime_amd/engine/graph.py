@@ -94,7 +94,12 @@ class DecodeGraph:
                     return runner.model.forward(self.ctx, dev["ids"], self.cache_views, dev["rows"])
                 graph = torch.cuda.CUDAGraph()
                 torch.cuda.synchronize(runner.device)
-                with torch.cuda.graph(graph):
+                # all graphs of a runner take their buffers from one pool: only one of them runs
+                # at a time and its logits are consumed before the next step, so the memory they
+                # need is that of the largest, not the sum over batch sizes and buckets
+                if runner._graph_pool is None:
+                    runner._graph_pool = torch.cuda.graph_pool_handle()
+                with torch.cuda.graph(graph, pool=runner._graph_pool):
                     self.logits = runner.model.forward(self.ctx, dev["ids"], self.cache_views, dev["rows"])
                 self.graph = graph
         self.graph.replay()

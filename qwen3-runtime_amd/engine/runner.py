@@ -37,6 +37,7 @@ class ModelRunner:
         self.vocab_size = model.plan.vocab_size
         self.hip_graph = bool(hip_graph) and self.device.type == "cuda"
         self._graphs: dict[tuple, "_DecodeGraph"] = {}
+        self._graph_pool = None
         self._pinned: torch.Tensor | None = None
         self._copied = torch.cuda.Event() if self.device.type == "cuda" else None
         self.graph_max_batch = 256
