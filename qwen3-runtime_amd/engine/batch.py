@@ -62,25 +62,30 @@ def pack_step(entries: Sequence[StepEntry], cache, vocab_size: int, table_width:
     positions = np.empty(t, dtype=np.int32)
     seq_of_token = np.empty(t, dtype=np.int32)
     rows: list[int] = []
+    row_seq: list[int] = []
     for i, e in enumerate(entries):
         a, b = int(cu_q[i]), int(cu_q[i + 1])
         ids[a:b] = np.asarray(e.tokens, dtype=np.int64)
         positions[a:b] = np.arange(starts[i], starts[i] + q_lens[i], dtype=np.int32)
         seq_of_token[a:b] = i
         rows.extend(a + int(w) for w in e.want)
+        row_seq.extend(i for _ in e.want)
     if ids.min() < 0 or ids.max() >= vocab_size:
         raise ValueError(f"token id outside [0, {vocab_size})")
     kv_lens = [st + n for st, n in zip(starts, q_lens)]
     rids = [e.request_id for e in entries]
+    state_slots = np.asarray([cache.slots.slot(r) for r in rids], dtype=np.int32)
     arrays = {
         "ids": ids,
         "positions": positions,
         "seq_of_token": seq_of_token,
         "cu_q": cu_q,
         "kv_lens": np.asarray(kv_lens, dtype=np.int32),
-        "state_slots": np.asarray([cache.slots.slot(r) for r in rids], dtype=np.int32),
+        "state_slots": state_slots,
         "first_span": np.asarray([1 if st == 0 else 0 for st in starts], dtype=np.int32),
         "rows": np.asarray(rows, dtype=np.int32),
+        # the state slot of each wanted row's request (the sampler reads its options there)
+        "row_slots": state_slots[np.asarray(row_seq, dtype=np.int64)] if rows else np.zeros(0, dtype=np.int32),
     }
     width = table_width if table_width is not None else cache.table_width(rids)
     for gi in range(len(cache.groups)):

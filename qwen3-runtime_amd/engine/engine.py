@@ -93,8 +93,10 @@ class Engine:
         logits = self.runner.step(entries)
         tokens: list[int | None] = [None] * len(reqs)
         if sampling_reqs:
-            slot_rows = torch.tensor([self.cache.slots.slot(r.request_id) for r in sampling_reqs],
-                                     dtype=torch.int32, device=self.runner.device)
+            # the rows' state slots went up with the step's other arrays: no copy, no wait here
+            slot_rows = self.runner.last_row_slots
+            if slot_rows is None or slot_rows.numel() != len(sampling_reqs):
+                raise RuntimeError("the step's logits do not match the requests to sample for")
             sampled, logprobs = self.sampler.sample(logits, slot_rows, sampling_reqs)
             by_id = {r.request_id: (t, lp) for r, t, lp in zip(sampling_reqs, sampled, logprobs)}
             for i, req in enumerate(reqs):

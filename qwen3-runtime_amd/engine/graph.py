@@ -86,6 +86,7 @@ class DecodeGraph:
                     for st in runner.model.plan.order
                 ]
             dev = self.views_dev
+            runner.last_row_slots = dev["row_slots"]
             self.runs += 1
             with torch.inference_mode():
                 if self.runs < 2:
@@ -102,6 +103,7 @@ class DecodeGraph:
                 with torch.cuda.graph(graph, pool=runner._graph_pool):
                     self.logits = runner.model.forward(self.ctx, dev["ids"], self.cache_views, dev["rows"])
                 self.graph = graph
+        runner.last_row_slots = self.views_dev["row_slots"]
         self.graph.replay()
         return self.logits
 

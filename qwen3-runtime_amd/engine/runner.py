@@ -38,6 +38,8 @@ class ModelRunner:
         self.hip_graph = bool(hip_graph) and self.device.type == "cuda"
         self._graphs: dict[tuple, "_DecodeGraph"] = {}
         self._graph_pool = None
+        # device copy of the last step's "row_slots" (state slot of each row of the logits)
+        self.last_row_slots: torch.Tensor | None = None
         self._pinned: torch.Tensor | None = None
         self._copied = torch.cuda.Event() if self.device.type == "cuda" else None
         self.graph_max_batch = 256
@@ -58,6 +60,7 @@ class ModelRunner:
         else:
             packed = pack_step(entries, self.cache, self.vocab_size)
             dev = self._upload(packed)
+            self.last_row_slots = dev["row_slots"]
             logits = self._forward(packed, dev)
         for e in entries:
             self.cache.commit(e.request_id, len(e.tokens))
@@ -137,7 +140,9 @@ class ModelRunner:
         key = DecodeGraph.key_for(len(entries), max_kv, all(len(e.want) == 1 for e in entries))
         if key is None:
             packed = pack_step(entries, self.cache, self.vocab_size)
-            return self._forward(packed, self._upload(packed))
+            dev = self._upload(packed)
+            self.last_row_slots = dev["row_slots"]
+            return self._forward(packed, dev)
         graph = self._graphs.get(key)
         if graph is None:
             graph = DecodeGraph(self, key)

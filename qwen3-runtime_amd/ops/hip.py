@@ -502,7 +502,8 @@ class HipOps:
         """One token per row of ``logits``. Options are read from the row's state slot:
         ``fparams[slot]`` = temperature, top_p, min_p, repetition, presence, frequency;
         ``iparams[slot]`` = top_k; ``seeds[slot]`` = seed, index of the next draw (advanced
-        here). Returns (token int32 [R], logprob float32 [R], processed logits [R, V])."""
+        here). Returns (token int32 [R], logprob float32 [R], processed logits [R, V], buffer); the
+        first two are the rows of the int32 buffer [2, R], so that one copy brings both to the host."""
         _need(logits, "logits", torch.float32)
         r, v = logits.shape
         _need(slot, "slot", torch.int32, (r,))
@@ -513,8 +514,9 @@ class HipOps:
         if counts is not None:
             _need(counts, "counts", torch.int32, (n, v))
         work = torch.empty_like(logits)
-        tok = torch.empty((r,), dtype=torch.int32, device=logits.device)
-        lp = torch.empty((r,), dtype=torch.float32, device=logits.device)
+        # ids and log-probabilities side by side, so that one copy brings both to the host
+        both = torch.empty((2, r), dtype=torch.int32, device=logits.device)
+        tok, lp = both[0], both[1].view(torch.float32)
         a = _SampleArgs()
         a.logits, a.work, a.counts, a.slot = logits.data_ptr(), work.data_ptr(), _addr(counts), slot.data_ptr()
         a.fparams, a.iparams, a.seeds = fparams.data_ptr(), iparams.data_ptr(), seeds.data_ptr()
@@ -526,7 +528,7 @@ class HipOps:
             partials = torch.empty((r, parts, 4), dtype=torch.float32, device=logits.device)
             a.partials, a.parts = partials.data_ptr(), parts
         self._check(self.lib, self.lib.qrt_sample(byref(a), _stream()))
-        return tok, lp, work
+        return tok, lp, work, both
 
     def count_tokens(self, counts, slots, tokens):
         _need(counts, "counts", torch.int32)

@@ -56,8 +56,8 @@ class Sampler:
             self.ops.add_bias(logits, rows, toks, vals)
         forced = [r.next_forced_token() for r in reqs]
         any_forced = any(f is not None for f in forced)
-        tok, lp, work = self.ops.sample(logits, slot_rows, self.fparams, self.iparams, self.seeds, self.counts,
-                                        keep_processed=any_forced)
+        tok, lp, work, both = self.ops.sample(logits, slot_rows, self.fparams, self.iparams, self.seeds,
+                                              self.counts, keep_processed=any_forced)
         if any_forced:
             # teacher forcing: the given id, scored under the processed logits
             # (reference: qwen3_runtime/sampling.py:319-325)
@@ -68,4 +68,5 @@ class Sampler:
                     lp[i] = logp[i, int(f)]
         if self.counts is not None:
             self.ops.count_tokens(self.counts, slot_rows, tok)
-        return tok.tolist(), lp.tolist()
+        host = both.cpu()  # ids and log-probabilities in one copy, one wait
+        return host[0].tolist(), host[1].view(torch.float32).tolist()
