@@ -242,6 +242,11 @@ class CacheManager:
         """``page * page_size + offset`` of positions ``start .. start+n-1``
         (reference: qwen3_runtime/engine/block_manager.py:264-270)."""
         g = self.groups[group]
+        if n == 1:  # a decoded token: no arrays needed
+            page = g.tables[rid][start // g.page_size]
+            if page < 0:
+                raise AssertionError(f"request {rid!r} writes to a position whose page was given back")
+            return np.asarray([page * g.page_size + start % g.page_size], dtype=np.int32)
         pos = np.arange(start, start + n, dtype=np.int64)
         table = np.asarray(g.tables[rid], dtype=np.int64)
         pages = table[pos // g.page_size]

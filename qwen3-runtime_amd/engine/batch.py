@@ -58,18 +58,27 @@ def pack_step(entries: Sequence[StepEntry], cache, vocab_size: int, table_width:
     t = int(sum(q_lens))
     cu_q = np.zeros(s + 1, dtype=np.int32)
     np.cumsum(q_lens, out=cu_q[1:])
-    ids = np.empty(t, dtype=np.int32)
-    positions = np.empty(t, dtype=np.int32)
-    seq_of_token = np.empty(t, dtype=np.int32)
     rows: list[int] = []
     row_seq: list[int] = []
-    for i, e in enumerate(entries):
-        a, b = int(cu_q[i]), int(cu_q[i + 1])
-        ids[a:b] = np.asarray(e.tokens, dtype=np.int64)
-        positions[a:b] = np.arange(starts[i], starts[i] + q_lens[i], dtype=np.int32)
-        seq_of_token[a:b] = i
-        rows.extend(a + int(w) for w in e.want)
-        row_seq.extend(i for _ in e.want)
+    if t == s:  # one token each (decoding): no loops over tokens
+        ids = np.asarray([e.tokens[0] for e in entries], dtype=np.int64).astype(np.int32)
+        positions = np.asarray(starts, dtype=np.int32)
+        seq_of_token = np.arange(s, dtype=np.int32)
+        for i, e in enumerate(entries):
+            if len(e.want):
+                rows.append(i)
+                row_seq.append(i)
+    else:
+        ids = np.empty(t, dtype=np.int32)
+        positions = np.empty(t, dtype=np.int32)
+        seq_of_token = np.empty(t, dtype=np.int32)
+        for i, e in enumerate(entries):
+            a, b = int(cu_q[i]), int(cu_q[i + 1])
+            ids[a:b] = np.asarray(e.tokens, dtype=np.int64)
+            positions[a:b] = np.arange(starts[i], starts[i] + q_lens[i], dtype=np.int32)
+            seq_of_token[a:b] = i
+            rows.extend(a + int(w) for w in e.want)
+            row_seq.extend(i for _ in e.want)
     if ids.min() < 0 or ids.max() >= vocab_size:
         raise ValueError(f"token id outside [0, {vocab_size})")
     kv_lens = [st + n for st, n in zip(starts, q_lens)]

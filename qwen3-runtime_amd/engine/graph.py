@@ -45,9 +45,22 @@ class DecodeGraph:
         self.copied = torch.cuda.Event()
         self.ctx = None
         self.runs = 0
+        # what the host buffer holds: the requests of the last fill and their lengths before it
+        self._last_rids: list | None = None
+        self._last_starts: list[int] | None = None
+        self._host_views = None
+        self._row_index = None
 
     def _fill(self, entries: Sequence[StepEntry]):
         runner = self.runner
+        rids = [e.request_id for e in entries]
+        starts = [runner.cache.length(r) for r in rids]
+        if (self.graph is not None and rids == self._last_rids
+                and all(a == b + 1 for a, b in zip(starts, self._last_starts))):
+            self._fill_next(entries, rids, starts)
+            self._last_starts = starts
+            return None
+        self._last_rids, self._last_starts = rids, starts
         packed = pack_step(entries, runner.cache, runner.vocab_size, table_width=self.width)
         if self.layout is None:
             off, layout = 0, []
@@ -68,6 +81,41 @@ class DecodeGraph:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
         return packed
+
+    def _fill_next(self, entries: Sequence[StepEntry], rids, starts) -> None:
+        """The same requests one token further (the usual decode step): the host buffer is brought
+        up to date in place. New ids, positions and lengths one up, the slots of the new positions,
+        and a block-table entry where a request has begun a page; groups with a window (whose
+        pages are given back as the window passes) get their tables written afresh."""
+        cache = self.runner.cache
+        self.copied.synchronize()  # the previous copy has left the host buffer
+        if self._host_views is None:
+            host = self.host.numpy()
+            self._host_views = {name: host[off: off + int(np.prod(shape))].reshape(shape)
+                                for name, off, shape in self.layout}
+            self._row_index = np.arange(self.batch)
+        view = self._host_views
+        ids = np.asarray([e.tokens[0] for e in entries], dtype=np.int64)
+        if ids.min() < 0 or ids.max() >= self.runner.vocab_size:
+            raise ValueError(f"token id outside [0, {self.runner.vocab_size})")
+        view["ids"][:] = ids
+        pos = np.asarray(starts, dtype=np.int64)
+        view["positions"][:] = pos
+        view["kv_lens"][:] = pos + 1
+        for gi, g in enumerate(cache.groups):
+            table = view[f"table{gi}"]
+            page_index = pos // g.page_size
+            if g.window is not None:
+                cache.fill_tables(gi, rids, table)
+            else:
+                for i in np.nonzero(pos % g.page_size == 0)[0]:
+                    table[i, page_index[i]] = g.tables[rids[i]][page_index[i]]
+            pages = table[self._row_index, page_index].astype(np.int64)
+            if (pages < 0).any():
+                raise AssertionError("a request writes to a position whose page was given back")
+            view[f"slots{gi}"][:] = pages * g.page_size + pos % g.page_size
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
 
     def _views(self):
         return {name: self.dev[off: off + int(np.prod(shape))].view(shape) for name, off, shape in self.layout}
