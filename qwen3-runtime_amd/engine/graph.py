@@ -18,6 +18,7 @@ from typing import Sequence
 import numpy as np
 import torch
 
+from ..cache.pages import CacheFull
 from .batch import StepEntry, pack_step
 
 MIN_BUCKET = 512
@@ -55,11 +56,12 @@ class DecodeGraph:
         runner = self.runner
         rids = [e.request_id for e in entries]
         starts = [runner.cache.length(r) for r in rids]
-        if (self.graph is not None and rids == self._last_rids
-                and all(a == b + 1 for a, b in zip(starts, self._last_starts))):
-            self._fill_next(entries, rids, starts)
-            self._last_starts = starts
-            return None
+        if self.graph is not None and rids == self._last_rids:
+            if starts != self._last_starts and all(a == b + 1 for a, b in zip(starts, self._last_starts)):
+                self._advance(rids, starts)
+            if starts == self._last_starts:  # the buffer holds this step, but for the ids
+                self._send(entries)
+                return None
         self._last_rids, self._last_starts = rids, starts
         packed = pack_step(entries, runner.cache, runner.vocab_size, table_width=self.width)
         if self.layout is None:
@@ -82,23 +84,23 @@ class DecodeGraph:
         self.copied.record()
         return packed
 
-    def _fill_next(self, entries: Sequence[StepEntry], rids, starts) -> None:
-        """The same requests one token further (the usual decode step): the host buffer is brought
-        up to date in place. New ids, positions and lengths one up, the slots of the new positions,
-        and a block-table entry where a request has begun a page; groups with a window (whose
-        pages are given back as the window passes) get their tables written afresh."""
-        cache = self.runner.cache
-        self.copied.synchronize()  # the previous copy has left the host buffer
+    def _host(self):
         if self._host_views is None:
             host = self.host.numpy()
             self._host_views = {name: host[off: off + int(np.prod(shape))].reshape(shape)
                                 for name, off, shape in self.layout}
             self._row_index = np.arange(self.batch)
-        view = self._host_views
-        ids = np.asarray([e.tokens[0] for e in entries], dtype=np.int64)
-        if ids.min() < 0 or ids.max() >= self.runner.vocab_size:
-            raise ValueError(f"token id outside [0, {self.runner.vocab_size})")
-        view["ids"][:] = ids
+        return self._host_views
+
+    def _advance(self, rids, starts) -> None:
+        """The same requests one token further (the usual decode step): the host buffer is brought
+        up to date in place, but for the ids. Positions and lengths one up, the slots of the new
+        positions, and a block-table entry where a request has begun a page; groups with a window
+        (whose pages are given back as the window passes) get their tables written afresh. The
+        pages of the new positions must be reserved."""
+        cache = self.runner.cache
+        self.copied.synchronize()  # the previous copy has left the host buffer
+        view = self._host()
         pos = np.asarray(starts, dtype=np.int64)
         view["positions"][:] = pos
         view["kv_lens"][:] = pos + 1
@@ -114,8 +116,37 @@ class DecodeGraph:
             if (pages < 0).any():
                 raise AssertionError("a request writes to a position whose page was given back")
             view[f"slots{gi}"][:] = pages * g.page_size + pos % g.page_size
+        self._last_starts = list(starts)
+
+    def _send(self, entries: Sequence[StepEntry]) -> None:
+        """Write the step's ids into the host buffer and start its copy to the device."""
+        ids = np.asarray([e.tokens[0] for e in entries], dtype=np.int64)
+        if ids.min() < 0 or ids.max() >= self.runner.vocab_size:
+            raise ValueError(f"token id outside [0, {self.runner.vocab_size})")
+        self._host()["ids"][:] = ids
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
+
+    def prepare_next(self) -> None:
+        """Called when the step just launched has been entered into the cache's books: while the
+        GPU runs it, get the buffer ready for the step that most often follows, the same requests
+        one token further. Their pages are reserved now, in the order the scheduler would; if one
+        cannot get its page, or would leave this graph's bucket, nothing is prepared. A request
+        that ends instead gives its page back with all its others."""
+        if self.graph is None or self._last_rids is None:
+            return
+        cache, rids = self.runner.cache, self._last_rids
+        starts = [cache.length(r) for r in rids]
+        if any(a != b + 1 for a, b in zip(starts, self._last_starts)):
+            return
+        if max(starts) + 1 > min(self.bucket, self.runner.max_model_len):
+            return
+        try:
+            for r in rids:
+                cache.reserve(r, 1)
+        except CacheFull:
+            return
+        self._advance(rids, starts)
 
     def _views(self):
         return {name: self.dev[off: off + int(np.prod(shape))].view(shape) for name, off, shape in self.layout}

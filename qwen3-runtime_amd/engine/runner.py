@@ -55,8 +55,9 @@ class ModelRunner:
         for e in entries:
             self.cache.reserve(e.request_id, len(e.tokens))
         pure_decode = all(len(e.tokens) == 1 for e in entries)
+        graph = None
         if self.hip_graph and pure_decode and len(entries) <= self.graph_max_batch:
-            logits = self._step_graph(entries)
+            logits, graph = self._step_graph(entries)
         else:
             packed = pack_step(entries, self.cache, self.vocab_size)
             dev = self._upload(packed)
@@ -64,6 +65,8 @@ class ModelRunner:
             logits = self._forward(packed, dev)
         for e in entries:
             self.cache.commit(e.request_id, len(e.tokens))
+        if graph is not None:
+            graph.prepare_next()  # host work for the next step while the GPU runs this one
         return logits
 
     # ---- eager path ----------------------------------------------------------
@@ -142,9 +145,9 @@ class ModelRunner:
             packed = pack_step(entries, self.cache, self.vocab_size)
             dev = self._upload(packed)
             self.last_row_slots = dev["row_slots"]
-            return self._forward(packed, dev)
+            return self._forward(packed, dev), None
         graph = self._graphs.get(key)
         if graph is None:
             graph = DecodeGraph(self, key)
             self._graphs[key] = graph
-        return graph.run(entries)
+        return graph.run(entries), graph

@@ -106,12 +106,13 @@ def test_preemption_does_not_change_tokens(model_folders):
     assert m.engine.cache.num_free_pages == 12 and m.engine.cache.slots.num_free == 3
 
 
-@pytest.mark.parametrize("seed,graph", [(0, False), (1, True), (2, False)])
+@pytest.mark.parametrize("seed,graph", [(0, False), (0, True), (1, True), (2, False), (2, True), (3, True)])
 def test_random_traffic_with_few_pages(model_folders, seed, graph):
     """Requests of random lengths arriving at random steps into a pool too small for them:
     portions, decoding, waiting, preemption and recomputation in every order the seed gives.
     Every request ends with the tokens it gets when it runs alone; after every step no page is
-    lost or held twice, and at the end all pages and slots are free."""
+    lost or held twice, and at the end all pages and slots are free. With graphs, decode steps
+    also reserve the next step's pages ahead, which must change none of this."""
     import random
 
     rng = random.Random(seed)
