@@ -321,7 +321,6 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
 // lanes that read one MFMA operand together hit 16 different groups of banks.
 constexpr int KROW = D + 8;                // elements per key row in LDS
 constexpr int VROW = 40;                   // elements per value row (one head element, 32 keys) in LDS
-constexpr int PIECES = (4 * D + 255) / 256;  // 16-byte pieces per thread per operand and block
 constexpr int STAGE_ELEMS = 32 * KROW + D * VROW;
 
 template <int RT, bool P2>
@@ -392,81 +391,76 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
     for (int i = 0; i < DB; ++i) o[t][i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   }
 
-  // Block table entries are looked up one round before the loads that need them, so that no
-  // load waits for another: lookup(b + 2) and fetch(b + 1) are in flight while block b is multiplied.
+  // Who fetches what. A block of 32 keys is four groups of 8 consecutive keys, one per wave.
+  // Pages hold a multiple of 8 keys, so a group lies in one page: the wave needs ONE block-table
+  // entry per block, found with scalar instructions, for its keys (8 rows of D elements, one
+  // contiguous piece of memory) and for the same 8 keys of the transposed values (one 16-byte
+  // piece per head element). Entries are looked up one round before the loads that need them:
+  // lookup(b + 2) and fetch(b + 1) are in flight while block b is multiplied. Every load is
+  // unconditional (the group's first key is clamped into pages the sequence holds; what lies
+  // outside is masked with the scores or zeroed by a select): with loads under branches the
+  // compiler can no longer count which are in flight and waits for all of them in the middle of
+  // the products.
   const size_t page_stride = (size_t)a.nkv * ps * D;  // elements per page, keys and values alike
   const bf16_t* k_head = a.k_cache + (size_t)kvh * ps * D;
   const bf16_t* v_head = a.v_cache + (size_t)kvh * D * ps;
-  bf16x8_t kpiece[PIECES], vpiece[PIECES];
-  // Every load below is unconditional (indices are clamped into pages the sequence holds, what
-  // lies outside is zeroed by a select): with loads under branches the compiler can no longer
-  // count which are in flight and waits for all of them in the middle of the products.
-  constexpr bool ALL_THREADS = (4 * D) % 256 == 0;  // every thread has PIECES pieces
-  auto lookup = [&](int b, int* kpage, int* vpage) {
-    const int base = b << 5;
+  const int w8 = 8 * __builtin_amdgcn_readfirstlane(wave);  // this wave's group within a block
+  constexpr int LANE_PIECES = (D + 63) / 64;   // 16-byte pieces per lane, of keys and of values
+  constexpr bool ALL_LANES = D % 64 == 0;
+  bf16x8_t kpiece[LANE_PIECES], vpiece[LANE_PIECES];
+  auto group_start = [&](int b) { return min(max((b << 5) + w8, lo & ~7), blk_pos_max & ~7); };
+  auto lookup = [&](int b) { return table[page_div<P2>(group_start(b), ps, psh)]; };
+  auto fetch = [&](int b, int page) {  // global -> registers
+    const int off = page_mod<P2>(group_start(b), ps);
+    const bf16_t* kp = k_head + (size_t)page * page_stride + (size_t)off * D;  // 8 keys: 8 D elements in a row
+    const bf16_t* vp = v_head + (size_t)page * page_stride + off;
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      if (ALL_THREADS || c < 4 * D) {
-        const int kidx = min(max(base + c / (D / 8), lo), blk_pos_max);  // masked later where clamped
-        kpage[i] = table[page_div<P2>(kidx, ps, psh)];
-        const int kv0 = min(max(base + 8 * (c & 3), lo & ~7), blk_pos_max & ~7);
-        vpage[i] = table[page_div<P2>(kv0, ps, psh)];
-      }
-    }
-  };
-  auto fetch = [&](int b, const int* kpage, const int* vpage) {  // global -> registers: this thread's pieces of block b
-    const int base = b << 5;
-#pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      if (ALL_THREADS || c < 4 * D) {
-        const int key = c / (D / 8), part = c - key * (D / 8);
-        const int kidx = min(max(base + key, lo), blk_pos_max);
-        kpiece[i] = *(const bf16x8_t*)(k_head + (size_t)kpage[i] * page_stride + (page_mod<P2>(kidx, ps) * D + 8 * part));
-        const int d = c >> 2, kv0 = min(max(base + 8 * (c & 3), lo & ~7), blk_pos_max & ~7);
-        vpiece[i] = *(const bf16x8_t*)(v_head + (size_t)vpage[i] * page_stride + (d * ps + page_mod<P2>(kv0, ps)));
+    for (int i = 0; i < LANE_PIECES; ++i) {
+      const int c = lane + 64 * i;
+      if (ALL_LANES || c < D) {
+        kpiece[i] = *(const bf16x8_t*)(kp + 8 * c);
+        vpiece[i] = *(const bf16x8_t*)(vp + (size_t)c * ps);
       }
     }
   };
   auto stash = [&](int b, int stage) {  // registers -> LDS: block b into its stage
     bf16_t* kb = lds_kv + stage * STAGE_ELEMS;
     bf16_t* vb = kb + 32 * KROW;
-    const int base = b << 5;
+    // values of keys no row of the block sees were read from a clamped place: they may be
+    // anything, and 0 * NaN is NaN, so they become zeros
+    const int g0 = (b << 5) + w8;
+    const bool seen = g0 <= blk_pos_max && g0 + 7 >= lo;
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      if (ALL_THREADS || c < 4 * D) {
-        const int key = c / (D / 8), part = c - key * (D / 8);
-        // row 16 s2 + r16 of the stage holds the key that lane r16 of sub-block s2 multiplies:
-        // the 16 lanes of an operand read 16 consecutive padded rows, all in different banks
-        const int row = 16 * ((key >> 2) & 1) + 4 * (key >> 3) + (key & 3);
+    for (int i = 0; i < LANE_PIECES; ++i) {
+      const int c = lane + 64 * i;
+      if (ALL_LANES || c < D) {
+        // keys: piece c of the group is key c / (D / 8) of it, elements 8 (c % (D / 8)) onward; row
+        // 16 s2 + r16 of the stage holds the key that lane r16 of sub-block s2 multiplies (key
+        // 8 q + 4 s2 + r of the block sits in row 16 s2 + 4 q + r), so that the 16 lanes of an
+        // operand read 16 consecutive padded rows, all in different banks
+        const int kl = c / (D / 8), part = c - kl * (D / 8);
+        const int row = 16 * (kl >> 2) + (w8 >> 1) + (kl & 3);
         *(bf16x8_t*)(kb + row * KROW + 8 * part) = kpiece[i];
-        const int d = c >> 2, j = c & 3;
-        // values of keys no row of the block sees were read from a clamped place: they may be
-        // anything, and 0 * NaN is NaN, so they become zeros
-        const int kv0 = base + 8 * j;
-        const bool seen = kv0 <= blk_pos_max && kv0 + 7 >= lo;
         bf16x8_t v = vpiece[i];
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = seen ? v[e] : (bf16_t)0.0f;
-        *(bf16x8_t*)(vb + d * VROW + 8 * j) = v;
+        *(bf16x8_t*)(vb + c * VROW + w8) = v;
       }
     }
   };
 
-  int kpage[PIECES], vpage[PIECES];
+  int page = 0;
   if (b0 < b1) {  // a split may be left without blocks
-    lookup(b0, kpage, vpage);
-    fetch(b0, kpage, vpage);
-    if (b0 + 1 < b1) lookup(b0 + 1, kpage, vpage);
+    page = lookup(b0);
+    fetch(b0, page);
+    if (b0 + 1 < b1) page = lookup(b0 + 1);
     stash(b0, 0);
   }
   __syncthreads();
   for (int b = b0; b < b1; ++b) {
     const int stage = (b - b0) & 1;
-    if (b + 1 < b1) fetch(b + 1, kpage, vpage);      // with the entries the last round looked up
-    if (b + 2 < b1) lookup(b + 2, kpage, vpage);     // in flight until the next round
+    if (b + 1 < b1) fetch(b + 1, page);       // with the entry the last round looked up
+    if (b + 2 < b1) page = lookup(b + 2);     // in flight until the next round
     if (b >= wb0 && b < wb1) {  // uniform over the wave
       const int base = b << 5;
       const bf16_t* kb = lds_kv + stage * STAGE_ELEMS;
