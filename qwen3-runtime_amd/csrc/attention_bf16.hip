@@ -449,13 +449,16 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
     }
   };
 
-  int page = 0;
-  if (b0 < b1) {  // a split may be left without blocks
-    page = lookup(b0);
-    fetch(b0, page);
-    if (b0 + 1 < b1) page = lookup(b0 + 1);
-    stash(b0, 0);
-  }
+  // The first block is fetched and stored on every path, also by a split that is left without
+  // blocks (it takes the sequence's last block and never looks at it): the wait for these
+  // loads then also settles, for the compiler, that the queries have arrived. Were it under a
+  // branch, the waits it places for the queries inside the loop would also wait for the loads
+  // of the block after next, in the middle of the products.
+  const int b_first = min(b0, all_b1 - 1);
+  int page = lookup(b_first);
+  fetch(b_first, page);
+  if (b0 + 1 < b1) page = lookup(b0 + 1);
+  stash(b_first, 0);
   __syncthreads();
   for (int b = b0; b < b1; ++b) {
     const int stage = (b - b0) & 1;
