@@ -41,6 +41,10 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill measurement")
+    ap.add_argument("--workload", default="decode", choices=["decode", "mix"],
+                    help="decode: the closed batch (default). mix: --requests requests with prompts of 128 to 4,096 "
+                         "tokens and 256 output tokens each through the scheduler, prompts read in portions of 2,048")
+    ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure only the 2,048-token prefill (for profiling); prints a reduced line")
     args = ap.parse_args()
@@ -62,11 +66,16 @@ def main() -> int:
     steps, warmup = args.steps, args.warmup
     page = 16
     max_batch = args.batch if (args.no_points or args.prefill_only) else max(args.batch, 64)
+    mix = args.workload == "mix"
+    if mix:
+        max_batch = args.requests
     budget = 2048  # tokens per step
     # a request decodes while later ones are still read in: up to this many steps before the timed ones
     lead = lambda batch: batch * -(-args.prompt_len // budget)
     per_req_tokens = args.prompt_len + steps + warmup + lead(max_batch) + 10
     pages = max_batch * (-(-per_req_tokens // page) + 1)
+    if mix:
+        pages = max_batch * (-(-(4096 + 256) // page) + 1)
     t0 = time.time()
     engine = build_engine(
         None, config=cfg, seed=20260825, dtype=args.dtype, block_size=page, num_kv_blocks=pages,
@@ -127,6 +136,35 @@ def main() -> int:
 
     if args.prefill_only:
         print(json.dumps({"metric": "prefill tok/s, one 2,048-token prompt", "prefill": prefill_run()}), flush=True)
+        return 0
+
+    if mix:
+        # continuous batching: every request queued at once, prompts read in portions beside the
+        # decoding of those already in
+        lengths = torch.randint(128, 4097, (args.requests,), generator=gen).tolist()
+        prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for n in lengths]
+        engine.generate_batch(prompts[:2], max_tokens=8)  # warm-up: libraries, allocator
+        torch.cuda.synchronize(dev)
+        t = time.perf_counter()
+        reqs = [engine.request(engine.add_request(p, max_tokens=256, sampling=SamplingParams())) for p in prompts]
+        n_steps = 0
+        while not engine.is_finished():
+            engine.step()
+            n_steps += 1
+        torch.cuda.synchronize(dev)
+        dt = time.perf_counter() - t
+        out_tokens = sum(len(r.output_tokens) for r in reqs)
+        print(json.dumps({
+            "metric": f"output tok/s, {args.requests} requests with 128-4,096-token prompts and 256 output tokens each, "
+                      f"continuous batching ({args.preset} shape)",
+            "value": round(out_tokens / dt, 1), "unit": "tok/s", "n_gpus": 1, "seconds": round(dt, 3),
+            "engine_steps": n_steps, "prompt_tokens": sum(lengths), "output_tokens": out_tokens,
+            "total_tok_per_s": round((sum(lengths) + out_tokens) / dt, 1),
+            "preemptions": engine.scheduler.num_preemptions, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: uniform-random token ids and lengths, seeded random weights",
+            "config": {"model": f"{args.preset} shape", "layers": cfg.num_hidden_layers, "max_num_seqs": max_batch,
+                       "max_num_batched_tokens": budget, "page_size": page, "hip_graph": not args.no_graph},
+        }), flush=True)
         return 0
 
     dt, kv_tokens = decode_run(args.batch, steps, warmup)
