@@ -148,18 +148,32 @@ def main() -> int:
         t = time.perf_counter()
         reqs = [engine.request(engine.add_request(p, max_tokens=256, sampling=SamplingParams())) for p in prompts]
         n_steps = 0
+        stamps: dict[int, list[float]] = {r.request_id: [] for r in reqs}  # arrival time of every token
         while not engine.is_finished():
-            engine.step()
+            out = engine.step()
+            now = time.perf_counter() - t
+            for rid, tok, _done in out:
+                if tok is not None:
+                    stamps[rid].append(now)
             n_steps += 1
         torch.cuda.synchronize(dev)
         dt = time.perf_counter() - t
         out_tokens = sum(len(r.output_tokens) for r in reqs)
+        # the reference's closed-batch figures (qwen3_runtime/serving/slo_harness.py:47-87): time to
+        # the first token, time per output token after it, gaps between consecutive tokens
+        ttft = sorted(ts[0] for ts in stamps.values())
+        tpot = sorted((ts[-1] - ts[0]) / (len(ts) - 1) for ts in stamps.values() if len(ts) > 1)
+        itl = sorted(b - a for ts in stamps.values() for a, b in zip(ts, ts[1:]))
+        pick = lambda xs, q: round(xs[min(len(xs) - 1, int(q * len(xs)))] * 1e3, 2) if xs else None
         print(json.dumps({
             "metric": f"output tok/s, {args.requests} requests with 128-4,096-token prompts and 256 output tokens each, "
                       f"continuous batching ({args.preset} shape)",
             "value": round(out_tokens / dt, 1), "unit": "tok/s", "n_gpus": 1, "seconds": round(dt, 3),
             "engine_steps": n_steps, "prompt_tokens": sum(lengths), "output_tokens": out_tokens,
             "total_tok_per_s": round((sum(lengths) + out_tokens) / dt, 1),
+            "ttft_ms": {"p50": pick(ttft, 0.5), "p99": pick(ttft, 0.99)},
+            "tpot_ms": {"p50": pick(tpot, 0.5), "p99": pick(tpot, 0.99)},
+            "itl_ms": {"p50": pick(itl, 0.5), "p99": pick(itl, 0.99)},
             "preemptions": engine.scheduler.num_preemptions, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: uniform-random token ids and lengths, seeded random weights",
             "config": {"model": f"{args.preset} shape", "layers": cfg.num_hidden_layers, "max_num_seqs": max_batch,

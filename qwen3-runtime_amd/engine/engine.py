@@ -30,6 +30,7 @@ class Engine:
         self.sampler = Sampler(self.runner.ops, self.cache.slots, self.runner.vocab_size, self.runner.device)
         self._requests: dict[int, Request] = {}
         self.last_step_stats: dict | None = None
+        self._fatal_error: str | None = None
 
     # ---- requests --------------------------------------------------------------
     def add_request(
@@ -42,6 +43,7 @@ class Engine:
         stop_token_ids: Sequence[int] = (),
         forced_tokens: Sequence[int] | None = None,
     ) -> int:
+        self._check_health()
         req = Request(token_ids, max_tokens, ignore_eos, sampling=sampling,
                       stop_token_ids=stop_token_ids, forced_tokens=forced_tokens)
         bad = [t for t in req.token_ids if not 0 <= t < self.runner.vocab_size]
@@ -65,7 +67,15 @@ class Engine:
         return self.scheduler.is_finished()
 
     # ---- one step -----------------------------------------------------------------
+    def _check_health(self) -> None:
+        """After a failure on the device side of a step the cache's books and the device's state
+        no longer agree: the engine refuses further work
+        (reference: qwen3_runtime/engine/engine.py:210-225)."""
+        if self._fatal_error is not None:
+            raise RuntimeError("engine terminated after a failed step: " + self._fatal_error)
+
     def step(self) -> list[tuple[int, int | None, bool]]:
+        self._check_health()
         preempt_before = self.scheduler.num_preemptions
         reqs = self.scheduler.schedule()
         if not reqs:
@@ -90,6 +100,13 @@ class Engine:
                 decode_tokens += n
             else:
                 prefill_tokens += n
+        try:
+            return self._run(reqs, entries, sampling_reqs, prefill_tokens, decode_tokens, preempt_before)
+        except BaseException as exc:
+            self._fatal_error = f"{type(exc).__name__}: {exc}"
+            raise
+
+    def _run(self, reqs, entries, sampling_reqs, prefill_tokens, decode_tokens, preempt_before):
         logits = self.runner.step(entries)
         tokens: list[int | None] = [None] * len(reqs)
         if sampling_reqs:

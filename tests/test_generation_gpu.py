@@ -139,6 +139,31 @@ def test_random_traffic_with_few_pages(model_folders, seed, graph):
     assert eng.cache.num_free_pages == 17 and eng.cache.slots.num_free == 4
 
 
+def test_engine_refuses_work_after_a_failed_step(model_folders):
+    """A step that fails on the device side (forced here from the host: the step function raises)
+    leaves cache and device in an unknown state; the engine then refuses steps and requests."""
+    from qwen3_runtime_amd.ops.hip import OpsError
+
+    cfg, _ = P.read_model(model_folders["tiny_a"])
+    eng = llm(model_folders["tiny_a"], page=16).engine
+    prompt = prompts_for(cfg, [9], seed=2)[0]
+    assert len(eng.generate(prompt, max_tokens=3)) == 3
+    eng.add_request(prompt, 4)
+    real = eng.runner.step
+
+    def failing(entries):
+        raise OpsError("attention: launch failed (forced by the test)")
+
+    eng.runner.step = failing
+    with pytest.raises(OpsError):
+        eng.step()
+    eng.runner.step = real
+    with pytest.raises(RuntimeError, match="engine terminated"):
+        eng.step()
+    with pytest.raises(RuntimeError, match="engine terminated"):
+        eng.add_request(prompt, 2)
+
+
 def test_decode_weight_copies_only_where_memory_allows(model_folders, capsys):
     from qwen3_runtime_amd.config.engine import EngineConfig
     from qwen3_runtime_amd.engine.factory import load
