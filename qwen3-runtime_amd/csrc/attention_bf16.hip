@@ -135,6 +135,70 @@ __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t*
   for (int i = 0; i < DB; ++i) o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[i], pb, o[i], 0, 0, 0);
 }
 
+// The same for RT tiles of a wave at once, step by step across the tiles instead of tile by
+// tile: the tiles' chains (scores -> maximum -> exponentials -> second product) do not depend
+// on each other, and written side by side in one stretch of code without branches between them
+// the exponentials of one tile can issue while the matrix pipe works on another's products.
+template <int RT>
+__device__ __forceinline__ void tiles_update(const f32x4_t (*sc)[2], const bf16x8_t* vv, const bool* whole, int base,
+                                             int quad, const bool* row_valid, const int* qpos, int window,
+                                             float scale_log2, float* m, float* l, f32x4_t (*o)[DB]) {
+  float s[RT][8];
+  bool any_masked = false;
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s[t][e] = sc[t][e >> 2][e & 3];
+    any_masked |= !whole[t];
+  }
+  if (any_masked) {  // the same for the whole wave
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = base + 8 * quad + e;
+        const bool vis = whole[t] || (row_valid[t] && key <= qpos[t] && (window == 0 || key > qpos[t] - window));
+        s[t][e] = vis ? s[t][e] : -INFINITY;
+      }
+  }
+  float m_use[RT], corr[RT];
+  bool moved = false;
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, s[t][e]);
+    mx = row_max4(mx);
+    const float m_new = fmaxf(m[t], mx * scale_log2);
+    m_use[t] = m_new == -INFINITY ? 0.f : m_new;
+    corr[t] = __builtin_amdgcn_exp2f(m[t] - m_use[t]);
+    m[t] = m_new;
+    moved |= corr[t] != 1.0f;
+  }
+  bf16x8_t pb[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pe = __builtin_amdgcn_exp2f(fmaf(s[t][e], scale_log2, -m_use[t]));
+      psum += pe;
+      pb[t][e] = (bf16_t)pe;
+    }
+    l[t] = l[t] * corr[t] + psum;
+  }
+  if (__any(moved)) {
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int i = 0; i < DB; ++i) o[t][i] *= corr[t];
+  }
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int t = 0; t < RT; ++t) o[t][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[i], pb[t], o[t][i], 0, 0, 0);
+}
+
 // ------------------------------------------------ keys and values straight from the pages
 struct KvBlock {  // the keys and values of one block of 32 keys, as MFMA operands
   bf16x8_t k[2][KFULL > 0 ? KFULL : 1];
@@ -483,9 +547,10 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
 #pragma unroll
       for (int i = 0; i < DB; ++i) vv[i] = *(const bf16x8_t*)(vb + (16 * i + r16) * VROW + 8 * quad);
 
+      f32x4_t sc[RT][2];
+      bool whole[RT];
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
-        f32x4_t sc[2];
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -493,11 +558,12 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
           for (int i = 0; i < KFULL; ++i)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk[s2][i], qreg[t][i], acc, 0, 0, 0);
           if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[s2], qtail[t], acc, 0, 0, 0);
-          sc[s2] = acc;
+          sc[t][s2] = acc;
         }
-        const bool whole = base + 31 <= tile_pos_min[t] && (a.window == 0 || base > tile_pos_max[t] - a.window);
-        tile_update(sc, vv, !whole, base, quad, row_valid[t], qpos[t], a.window, a.scale_log2, m[t], l[t], o[t]);
+        // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
+        whole[t] = base + 31 <= tile_pos_min[t] && (a.window == 0 || base > tile_pos_max[t] - a.window);
       }
+      tiles_update<RT>(sc, vv, whole, base, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
     }
     if (b + 1 < b1) stash(b + 1, stage ^ 1);
     __syncthreads();
