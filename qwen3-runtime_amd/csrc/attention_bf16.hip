@@ -812,9 +812,11 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
   QRT_CHECK((long long)a.num_tiles * a.nkv < (1ll << 31), "attention: %d tiles x %d key heads is too many blocks", a.num_tiles, a.nkv);
   dim3 grid(a.num_tiles * a.nkv, 1, a.num_splits), block(64 * a.waves);
-  if (a.row_tiles == 2 && a.waves == 4 && a.use_lds) {
-    const size_t smem = 2 * (size_t)STAGE_ELEMS * sizeof(bf16_t);
-    QRT_CHECK(smem <= 64 * 1024, "attention: head size %d needs %zu bytes of LDS", D, smem);
+  // the kernel that shares keys and values through LDS, where its two stages fit what a block
+  // may have without asking (64 KB: head sizes up to 208); the general kernel otherwise
+  constexpr size_t lds_bytes = 2 * (size_t)STAGE_ELEMS * sizeof(bf16_t);
+  if (a.row_tiles == 2 && a.waves == 4 && a.use_lds && lds_bytes <= 64 * 1024) {
+    const size_t smem = lds_bytes;
     if (p2) attention_bf16_prefill_kernel<2, true><<<grid, block, smem, stream>>>(a);
     else attention_bf16_prefill_kernel<2, false><<<grid, block, smem, stream>>>(a);
   } else if (a.row_tiles == 1 && p2) attention_bf16_kernel<1, true><<<grid, block, 0, stream>>>(a);

@@ -350,6 +350,7 @@ ATTN_CASES = [
     ([(1, 700)], 34, 2, 16, 32),
     ([(1, 100), (2, 61), (1, 24)], 4, 2, 32, 24),   # page sizes that are no power of two
     ([(20, 131), (300, 300)], 4, 1, 64, 40),
+    ([(150, 210)], 2, 1, 256, 16),                  # a long portion at a head size whose LDS stages do not fit
 ]
 
 
