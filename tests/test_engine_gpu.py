@@ -43,6 +43,35 @@ def test_cuttings_match_plain(model_folders, tiny_configs, name, cut, dtype):
     traces.compare(got, traces.plain_logits(model_folders[name], reqs), **TOL[dtype])
 
 
+@pytest.fixture(scope="module")
+def odd_folder(tmp_path_factory):
+    """A third tiny model with sizes the kernels' fast paths do not take: head size 80 (a 16-wide
+    remainder for the MFMA, no power of two for the wide q/k kernel), three query heads per key
+    head, a width, a feed-forward size and a vocabulary that are multiples of nothing much."""
+    from qwen3_runtime_amd.config.model import Qwen3Config
+    from qwen3_runtime_amd.weights import write_model_folder
+
+    cfg = Qwen3Config(vocab_size=333, hidden_size=176, num_hidden_layers=2, num_attention_heads=6,
+                      num_key_value_heads=2, head_dim=80, intermediate_size=208, rms_norm_eps=3e-6,
+                      rope_theta=50000.0, max_position_embeddings=512, tie_word_embeddings=True)
+    folder = tmp_path_factory.mktemp("odd")
+    write_model_folder(folder, cfg.to_dict(), seed=31)
+    return cfg, folder
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "portions", "mixed"])
+def test_odd_sizes_and_pages_of_24(odd_folder, cut, dtype):
+    """Pages of 24 tokens (no power of two: the kernels divide instead of shifting)."""
+    cfg, folder = odd_folder
+    page = 24
+    reqs = traces.make_requests(cfg.vocab_size, [5, 50, 97, 130], seed=2)
+    steps = getattr(traces, cut)(reqs)
+    loaded = load_gpu(folder, page, -(-traces.peak_tokens(steps, unit=72) // page), dtype)
+    got = traces.replay(loaded, steps)
+    traces.compare(got, traces.plain_logits(folder, reqs), **TOL[dtype])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_mixed_with_page_reuse(model_folders, tiny_configs, dtype):
     cfg, page = tiny_configs["tiny_b"]
