@@ -414,6 +414,38 @@ def test_long_portions_split_over_blocks_agree(ops, seqs, nq, nkv, d, ps, window
         close(got, want, 2e-2, 2e-2)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_paged_attention_random_shapes(ops, seed):
+    """Seeded random mixes of decoded tokens, short and long portions, head counts, head sizes,
+    page sizes, windows and key splits against the plain reference: every kernel variant and the
+    edges between them (16, 64 rows; blocks of 32 keys; pages) get hit by some seed."""
+    import random
+
+    rng = random.Random(1000 + seed)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+    nkv = rng.choice([1, 2, 3, 8])
+    g = rng.choice([1, 2, 3, 4, 5, 8])
+    nq = nkv * g
+    ps = rng.choice([8, 16, 24, 32, 40, 64])
+    kind = rng.choice(["decode", "short", "long", "mixed"])
+    seqs = []
+    for _ in range(rng.randint(1, 5)):
+        k = kind if kind != "mixed" else rng.choice(["decode", "short", "long"])
+        ql = {"decode": 1, "short": rng.randint(2, 20), "long": rng.randint(30, 260)}[k]
+        seqs.append((ql, ql + rng.choice([0, 0, rng.randint(1, 40), rng.randint(100, 700)])))
+    window = rng.choice([None, None, rng.randint(1, 300)])
+    splits = rng.choice([None, None, rng.randint(2, 9)])
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, seed=seed, window=window)
+    scale = 1.0 / math.sqrt(d)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, scale, window)
+    if splits:
+        ctx.scratch["attn_splits"] = splits
+    got = ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, window)
+    assert torch.isfinite(got.float()).all(), (seqs, nq, nkv, d, ps, window, splits)
+    close(got, want, 2e-2, 2e-2)
+
+
 def test_decode_attention_many_sequences_and_repeated_launches(ops):
     """Many sequences of very different lengths, launched again and again with other split counts."""
     g = torch.Generator().manual_seed(5)
