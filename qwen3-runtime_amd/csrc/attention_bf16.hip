@@ -63,6 +63,10 @@ struct AttnTileArgs {
   float scale_log2;
   int row_tiles;  // tiles of 16 rows per wave (general kernel): 1, 2 or 4
   int use_lds;    // long portions: share keys and values of a block of waves through LDS
+  // a launch that covers only some of the step's sequences (the others go to another kernel):
+  // the tokens whose rows the merge of key splits may write; null: all rows
+  const int* merge_tokens;
+  int num_merge_tokens;
 };
 
 constexpr int D = QRT_HEAD_DIM;
@@ -599,8 +603,10 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
 
 // out[row] = sum_s 2^(lse_s - M) O_s / sum_s 2^(lse_s - M); empty splits weigh 0
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
-                                       bf16_t* __restrict__ out, int num_splits) {
-  const size_t row = blockIdx.x;
+                                       bf16_t* __restrict__ out, int num_splits, const int* __restrict__ tokens,
+                                       int nq) {
+  // rows are (token, query head); with a token list the grid walks the listed tokens' rows only
+  const size_t row = tokens ? (size_t)tokens[blockIdx.x / nq] * nq + blockIdx.x % nq : blockIdx.x;
   const float* lse = part_lse + row * num_splits;
   float mx = -INFINITY;
   for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, lse[s]);
@@ -668,9 +674,10 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, quad = lane >> 4;
-  // every sequence is one tile here, so the tile list is not read: one dependent load less
-  // before the first key arrives
-  const int seq = blockIdx.x;
+  // every sequence is one tile here, so without a list the block's number is the sequence's: one
+  // dependent load less before the first key arrives. A list names the sequences of a launch
+  // that covers only some of the step's.
+  const int seq = a.tile_seq ? a.tile_seq[blockIdx.x] : blockIdx.x;
   const int kvh = blockIdx.y, split = blockIdx.z;
   const int g = a.nq / a.nkv;
   const int q_begin = a.cu_q[seq];
@@ -769,8 +776,8 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
   }
 }
 
-// every sequence at most 16 rows (max_q_len * g <= 16) and D <= 256; num_tiles = number of
-// sequences, the tile lists are not read
+// every listed sequence at most 16 rows (q_len * g <= 16) and D <= 256; num_tiles = number of
+// sequences; tile_seq lists them, or is null for all sequences of the step in order
 extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_total, hipStream_t stream) {
   AttnTileArgs a = *args;
   QRT_CHECK(a.nq > 0 && a.nkv > 0 && a.nq % a.nkv == 0, "attention: %d query heads do not divide into %d key heads",
@@ -789,8 +796,10 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   else attention_bf16_decode_kernel<false><<<grid, block, smem, stream>>>(a);
   QRT_LAUNCH_CHECK("attention_bf16_decode");
   if (a.num_splits > 1) {
-    attention_merge_kernel<<<dim3(num_rows_total), dim3(D >= 64 ? 64 : 32), 0, stream>>>(a.part_o, a.part_lse, a.out,
-                                                                                         a.num_splits);
+    const int merge_rows = a.merge_tokens ? a.num_merge_tokens * a.nq : num_rows_total;
+    if (merge_rows > 0)
+      attention_merge_kernel<<<dim3(merge_rows), dim3(D >= 64 ? 64 : 32), 0, stream>>>(
+          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq);
     QRT_LAUNCH_CHECK("attention_merge");
   }
   return 0;
@@ -828,8 +837,10 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   else return qrt_fail("attention: %d row tiles per wave at head size %d is not built", a.row_tiles, D);
   QRT_LAUNCH_CHECK("attention_bf16");
   if (a.num_splits > 1) {
-    attention_merge_kernel<<<dim3(num_rows_total), dim3(D >= 64 ? 64 : 32), 0, stream>>>(a.part_o, a.part_lse, a.out,
-                                                                                         a.num_splits);
+    const int merge_rows = a.merge_tokens ? a.num_merge_tokens * a.nq : num_rows_total;
+    if (merge_rows > 0)
+      attention_merge_kernel<<<dim3(merge_rows), dim3(D >= 64 ? 64 : 32), 0, stream>>>(
+          a.part_o, a.part_lse, a.out, a.num_splits, a.merge_tokens, a.nq);
     QRT_LAUNCH_CHECK("attention_merge");
   }
   return 0;

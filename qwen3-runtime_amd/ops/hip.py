@@ -64,6 +64,7 @@ class _AttnTileArgs(Structure):
         ("table_width", c_int), ("num_tiles", c_int), ("nq", c_int), ("nkv", c_int),
         ("page_size", c_int), ("window", c_int), ("num_splits", c_int), ("waves", c_int),
         ("scale_log2", c_float), ("row_tiles", c_int), ("use_lds", c_int),
+        ("merge_tokens", c_void_p), ("num_merge_tokens", c_int),
     ]
 
 
@@ -407,7 +408,8 @@ class HipOps:
     resident_blocks = 512  # blocks of the prompt kernels the chip holds at once: 2 on each of 256 CUs
 
     @staticmethod
-    def plan_tiles(q_lens, kv_lens, group_size: int, rows_per_tile: int, nkv: int = 1, resident: int = 0):
+    def plan_tiles(q_lens, kv_lens, group_size: int, rows_per_tile: int, nkv: int = 1, resident: int = 0,
+                   seq_ids=None):
         """Work list of the MFMA attention kernels: (sequence, first row) per tile of rows.
 
         Tiles that see the most keys come first: blocks that start late are then the short ones,
@@ -417,7 +419,8 @@ class HipOps:
         to end, so the second half of the list is turned round and long tiles share a CU with
         short ones."""
         items = []
-        for s, (n, kv) in enumerate(zip(q_lens, kv_lens)):
+        for i, (n, kv) in enumerate(zip(q_lens, kv_lens)):
+            s = i if seq_ids is None else seq_ids[i]  # the lists may cover some of the step's sequences
             first = kv - n
             for r in range(0, n * group_size, rows_per_tile):
                 last_tok = min(n * group_size, r + rows_per_tile) - 1
@@ -445,30 +448,67 @@ class HipOps:
         blocks = (max_kv + 31) // 32
         return max(1, min((256 + work - 1) // work, blocks // 8, 64))
 
+    # mixed steps: sequences with few rows leave the prompt kernel when their context is this long
+    split_launch_min_kv = 1024
+
     def _attention_mfma(self, q, out, cache, ctx, nq, nkv, d, scale, window):
+        """Which kernel for which sequences. Steps of decoded tokens only: the decode kernel.
+        Other steps: the prompt kernels; but sequences of at most 16 rows with a long context
+        (decoded tokens beside a prompt portion) would each walk all their keys in one block
+        there, and hold the step up, so they go to the decode kernel in a launch of their own,
+        which cuts their keys over many blocks."""
         if not scale > 0:
             raise OpsError(f"the bfloat16 attention kernels take a positive score scale, not {scale}")
+        g = nq // nkv
+        seqs = range(ctx.num_seqs)
+        if ctx.max_q_len * g <= 16 and d <= 256:
+            return self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, True)
+        small = [s for s in seqs if ctx.q_lens_host[s] * g <= 16]
+        if (d <= 256 and small and len(small) < ctx.num_seqs
+                and max(ctx.kv_lens_host[s] for s in small) >= self.split_launch_min_kv):
+            small_set = set(small)
+            big = [s for s in seqs if s not in small_set]
+            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, small, True)
+            self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, big, False)
+            return
+        self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False)
+
+    def _launch_attention(self, q, out, cache, ctx, nq, nkv, d, scale, window, subset, decode):
+        """One launch over the sequences in ``subset`` (None: all of the step's)."""
         lib = attention_library(d)
         g = nq // nkv
-        max_rows = ctx.max_q_len * g
-        decode = max_rows <= 16 and d <= 256
+        if subset is None:  # the step's own maxima: under a graph they are those of its bucket
+            q_lens, kv_lens = ctx.q_lens_host, ctx.kv_lens_host
+            max_rows, max_kv = ctx.max_q_len * g, ctx.max_kv_len
+        else:
+            q_lens = [ctx.q_lens_host[s] for s in subset]
+            kv_lens = [ctx.kv_lens_host[s] for s in subset]
+            max_rows, max_kv = max(q_lens) * g, max(kv_lens)
         waves = 1 if max_rows <= 16 else (2 if max_rows <= 32 else 4)
         # long portions: several row tiles per wave, so that loaded keys and values serve more rows
         row_tiles = 1 if max_rows <= 64 else (self.prefill_row_tiles if d <= 128 else min(2, self.prefill_row_tiles))
-        if decode:
-            tiles, n_tiles = None, ctx.num_seqs  # every sequence is one tile; the kernel needs no list
-        else:
-            key = ("attn_tiles", g, waves, row_tiles)
-            plan = ctx.scratch.get(key)
-            if plan is None:
-                host, n_tiles = self.plan_tiles(ctx.q_lens_host, ctx.kv_lens_host, g, 16 * waves * row_tiles, nkv,
-                                                self.resident_blocks if waves == 4 and row_tiles >= 2 else 0)
-                plan = (torch.from_numpy(host).to(q.device), n_tiles)
-                ctx.scratch[key] = plan
-            tiles, n_tiles = plan
+        key = ("attn_plan", g, decode, None if subset is None else tuple(subset))
+        plan = ctx.scratch.get(key)
+        if plan is None:  # the same for every layer of the step
+            dev = q.device
+            if decode:
+                tiles = None if subset is None else torch.tensor(subset, dtype=torch.int32, device=dev)
+                n_tiles = len(q_lens)
+            else:
+                host, n_tiles = self.plan_tiles(q_lens, kv_lens, g, 16 * waves * row_tiles, nkv,
+                                                self.resident_blocks if waves == 4 and row_tiles >= 2 else 0,
+                                                subset)
+                tiles = torch.from_numpy(host).to(dev)
+            tokens = None
+            if subset is not None:  # the tokens of these sequences: where a merge of key splits may write
+                cu = np.concatenate([[0], np.cumsum(ctx.q_lens_host)])
+                tokens = torch.from_numpy(np.concatenate([np.arange(cu[s], cu[s + 1]) for s in subset])
+                                          .astype(np.int32)).to(dev)
+            plan = (tiles, n_tiles, tokens)
+            ctx.scratch[key] = plan
+        tiles, n_tiles, tokens = plan
         splits = ctx.scratch.get("attn_splits") or (
-            self.choose_decode_splits(n_tiles, nkv, ctx.max_kv_len) if decode
-            else self.choose_splits(n_tiles, nkv, ctx.max_kv_len))
+            self.choose_decode_splits(n_tiles, nkv, max_kv) if decode else self.choose_splits(n_tiles, nkv, max_kv))
         a = _AttnTileArgs()
         a.q, a.out, a.k_cache, a.v_cache = q.data_ptr(), out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
         a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
@@ -476,7 +516,10 @@ class HipOps:
         a.block_table, a.table_width = cache.group.block_table.data_ptr(), cache.group.block_table.shape[1]
         if tiles is not None:
             a.tile_seq = tiles.data_ptr()
-            a.tile_row0 = tiles.data_ptr() + 4 * n_tiles
+            if not decode:
+                a.tile_row0 = tiles.data_ptr() + 4 * n_tiles
+        if tokens is not None:
+            a.merge_tokens, a.num_merge_tokens = tokens.data_ptr(), tokens.numel()
         a.num_tiles, a.nq, a.nkv, a.page_size, a.window = n_tiles, nq, nkv, cache.group.page_size, window
         a.num_splits, a.waves, a.row_tiles = splits, waves, row_tiles
         a.use_lds = 1 if self.prefill_through_lds else 0

@@ -446,6 +446,45 @@ def test_paged_attention_random_shapes(ops, seed):
     close(got, want, 2e-2, 2e-2)
 
 
+MIXED_CASES = [
+    # (seqs, nq, nkv, d, page, window): decoded tokens with a long context beside portions of prompts
+    ([(1, 1500), (200, 200), (1, 40), (1, 2100)], 8, 2, 128, 16, None),
+    ([(70, 900), (2, 1300), (1, 1), (3, 64)], 6, 2, 64, 24, None),
+    ([(1, 1200), (1, 700), (33, 33), (17, 500)], 4, 1, 32, 8, 300),
+    ([(16, 1100), (17, 1100)], 3, 3, 80, 16, None),   # one row count each side of the kernels' edge
+]
+
+
+@pytest.mark.parametrize("seqs,nq,nkv,d,ps,window", MIXED_CASES)
+def test_mixed_steps_go_through_two_launches_and_agree(ops, seqs, nq, nkv, d, ps, window, monkeypatch):
+    """A step with decoded tokens beside portions runs the decode kernel over the former and the
+    prompt kernels over the latter. Each launch writes its own tokens only, with any number of key
+    splits (the merge goes over the launch's tokens, not over all), and the result is the one
+    launch's too."""
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, seed=11, window=window)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, 0.125, window)
+    launches = []
+    inner = ops._launch_attention
+    monkeypatch.setattr(ops, "_launch_attention", lambda *a: (launches.append(a[-2:]), inner(*a))[1])
+    for min_kv, want_launches in ((1, 2), (1 << 30, 1)):
+        monkeypatch.setattr(ops, "split_launch_min_kv", min_kv)
+        for splits in (None, 1, 2, 5):
+            ctx.scratch.clear()
+            if splits:
+                ctx.scratch["attn_splits"] = splits
+            launches.clear()
+            got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 0.125, window)
+            assert len(launches) == want_launches, launches
+            close(got, want, 2e-2, 2e-2)
+    small = [s for s, (ql, _) in enumerate(seqs) if ql * (nq // nkv) <= 16]
+    monkeypatch.setattr(ops, "split_launch_min_kv", 1)
+    launches.clear()
+    ops.paged_attention(q, cache, ctx, nq, nkv, d, 0.125, window)
+    assert launches[0] == (small, True) and launches[1][1] is False
+    assert sorted(launches[0][0] + launches[1][0]) == list(range(len(seqs)))
+
+
 def test_decode_attention_many_sequences_and_repeated_launches(ops):
     """Many sequences of very different lengths, launched again and again with other split counts."""
     g = torch.Generator().manual_seed(5)
