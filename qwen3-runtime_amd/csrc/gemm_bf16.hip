@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 
 
 // ---------------------------------------------------------------- few rows
-// M <= 64 (decoding): the product is a stream of the weight matrix, so the
+// M <= 16 (decoding): the product is a stream of the weight matrix, so the
 // layout is chosen for memory parallelism, not for reuse. A block owns NT
 // tiles of 16 weight rows and all of K; its NW waves take the 32-wide k-steps
 // round-robin, so that in every round the block reads 16 rows x NW x 64
@@ -228,17 +228,9 @@ static int launch_skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtyp
 template <bool GATED>
 static int skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K, hipStream_t st) {
   const int tiles = (N + 15) / 16;
-  if (M <= 16) {
-    if (tiles >= 2048) return launch_skinny<1, 8, 2, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
-    if (tiles >= 512 || K < 4096) return launch_skinny<1, 8, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
-    return launch_skinny<1, 16, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
-  }
-  if (M <= 32) {
-    if (tiles >= 512) return launch_skinny<2, 8, 2, 4, GATED>(a, w, c, out_dtype, M, N, K, st);
-    return launch_skinny<2, 8, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
-  }
-  if (tiles >= 512 && !GATED) return launch_skinny<4, 8, 2, 2, GATED>(a, w, c, out_dtype, M, N, K, st);
-  return launch_skinny<4, 8, 1, 4, GATED>(a, w, c, out_dtype, M, N, K, st);
+  if (tiles >= 2048) return launch_skinny<1, 8, 2, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
+  if (tiles >= 512 || K < 4096) return launch_skinny<1, 8, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
+  return launch_skinny<1, 16, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
 }
 
 // Tile-major weights, M <= 16. Configurations from timing all of them on the shapes of the
@@ -251,6 +243,270 @@ static int skinny_tiled(const bf16_t* a, const bf16_t* w, void* c, int out_dtype
   if (!GATED && tiles >= 384 && k_parts == 1)
     return launch_skinny<1, 8, 2, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
   return launch_skinny<1, 8, 1, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st, k_parts);
+}
+
+__device__ __forceinline__ void store4(float* p, const float (&o)[4]) {
+  *(f32x4_t*)p = (f32x4_t){o[0], o[1], o[2], o[3]};
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float (&o)[4]) {
+  typedef bf16_t bf16x4_t __attribute__((ext_vector_type(4)));
+  *(bf16x4_t*)p = (bf16x4_t){(bf16_t)o[0], (bf16_t)o[1], (bf16_t)o[2], (bf16_t)o[3]};
+}
+
+// ---------------------------------------------------------------- 17 to 64 rows
+// Still a stream of the weight matrix, but the activations now weigh as much as the weights
+// if every wave fetches its own: four accumulator blocks of 16 rows want 4 KB of activations
+// for each KB of weights. So the waves that walk the same part of K (a K group) share the
+// activations through LDS: NWV waves side by side along N, NT tiles each, read one staged
+// copy, and the traffic for activations falls to MB / (NWV * NT) of the weights'. KW such
+// groups in a block take consecutive parts of the block's k-steps (the block's k-steps being
+// part blockIdx.y of all, as in the few-row kernel) and meet in LDS at the end, added in
+// group order. Weights, tile-major, go straight to registers, DEPTH chunks of KC k-steps
+// ahead; the activations of chunk c + 2 are fetched while chunk c is used and chunk c + 1
+// waits in the other LDS buffer, so there is one barrier per chunk. All loads are
+// unconditional, at clamped addresses: steps past the end are loaded again and count as zero.
+// Blocks start at different chunks of their k-steps and wrap round: every block reads all
+// the activations, and in step they would all ask the same L2 channels at the same time.
+// What a compute unit can pull through its memory pipeline is the limit (weights and
+// activations alike, about 55 GB/s each), so the row tiles are dealt out evenly over
+// gridDim.x blocks, chosen by the host as the number of compute units where there are more
+// tiles than that: a block gets floor or ceil of tiles / blocks, at most NWV * NT. A wave
+// without a tile reads a page of zeros instead, at no cost in memory traffic, and stores nothing.
+__device__ bf16x8_t qrt_zero_tile[64];
+
+template <int MB, int KW, int NWV, int NT, int KC, int DEPTH, bool GATED, typename TO>
+__global__ __launch_bounds__(64 * KW * NWV) void gemm_bf16_mid_kernel(const bf16_t* __restrict__ A,
+                                                                       const bf16_t* __restrict__ W,
+                                                                       TO* __restrict__ C, int M, int N, int K) {
+  constexpr int WT = GATED ? 2 * NT : NT;  // weight tiles per wave
+  constexpr int UPW = KC * MB / NWV;       // 1 KB units of activations a wave stages per chunk
+  static_assert(KC * MB % NWV == 0 && KC % 2 == 0, "the waves of a K group stage equal shares of a chunk");
+  static_assert(DEPTH == 1 || DEPTH == 2, "the weights run one or two chunks ahead");
+  extern __shared__ __align__(16) unsigned char smem_raw[];  // [KW][2] staged chunks
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kg = wave / NWV, nw = wave % NWV;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int ntiles = N >> 4;
+  const int tile_lo = (int)(blockIdx.x * (unsigned)ntiles / gridDim.x);  // N <= 2^20: no overflow
+  const int tile_hi = (int)((blockIdx.x + 1) * (unsigned)ntiles / gridDim.x);
+  const int tile0 = tile_lo + nw * NT;
+
+  // the k-steps of this block, then of this K group
+  // (K is a multiple of 64 here; parts and groups start at even k-steps: a cache line of
+  // activations holds two)
+  const int all_steps = K >> 5;
+  const int part = 2 * ((all_steps / 2 + gridDim.y - 1) / gridDim.y);
+  const int p0 = min(all_steps, (int)blockIdx.y * part), p1 = min(all_steps, p0 + part);
+  const int glen = 2 * (((p1 - p0) / 2 + KW - 1) / KW);
+  const int g0 = min(p1, p0 + kg * glen), g1 = min(p1, g0 + glen);
+  const int chunks = (glen + KC - 1) / KC;  // the same for every group: they share the barriers
+  const int last_step = all_steps - 1, last_pair = all_steps - 2;
+  const int rot = (int)((blockIdx.x * 5u + blockIdx.y * 3u + kg) % (unsigned)max(chunks, 1));
+  // first k-step of the c-th chunk in this block's order; past the last chunk nothing is live
+  auto chunk_start = [&](int c) {
+    int cc = c + rot;
+    if (cc >= chunks) cc -= chunks;
+    return c < chunks ? g0 + cc * KC : g1;
+  };
+
+  const bf16_t* wbase[WT];  // uniform over the wave: the lane is added at the load
+  int wstep[NT];            // elements from one k-step to the next: none in the page of zeros
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int tile = tile0 + t;
+    const bool mine = tile < tile_hi;
+    wstep[t] = mine ? 512 : 0;
+    wbase[t] = mine ? W + (size_t)tile * 16 * K : (const bf16_t*)qrt_zero_tile;
+    if (GATED) wbase[NT + t] = mine ? W + (size_t)(ntiles + tile) * 16 * K : (const bf16_t*)qrt_zero_tile;
+  }
+  // Staging of a chunk: unit u = (pair of k-steps u / (2 MB), row block (u / 2) % MB, half u % 2
+  // of its 16 rows); this wave stages units nw, nw + NWV, ... A unit is 8 rows x 128 bytes, whole
+  // cache lines: lane l reads row 8 half + l / 8, 16-byte piece l % 8 (k-step l % 8 / 4 of the
+  // pair, columns 8 (l % 4) .. + 7 of it). In LDS the piece of (k-step s, row block b, column
+  // group q, row i) lies at s * SS + b * BS + q * QS + 16 i bytes: the strides are padded so
+  // that the 8 pieces of a row, written together, fall into different banks, while the 16
+  // rows of a column group, read together, stay contiguous.
+  constexpr int QS = 256 + 16, BS = 4 * QS, SS = MB * BS + 64;  // bytes
+  const bf16_t* abase[UPW];
+  int apair[UPW], awrite[UPW];
+#pragma unroll
+  for (int j = 0; j < UPW; ++j) {
+    const int u = nw + NWV * j;
+    const int half = u % 2, b = (u / 2) % MB, piece = lane & 7, row = 8 * half + (lane >> 3);
+    apair[j] = 2 * (u / (2 * MB));
+    abase[j] = A + (size_t)min(16 * b + row, M - 1) * K + 8 * piece;
+    awrite[j] = (apair[j] + piece / 4) * SS + b * BS + (piece % 4) * QS + 16 * row;
+  }
+  unsigned char* group_buf = smem_raw + (size_t)kg * 2 * KC * SS;
+  const int aread = quad * QS + 16 * r16;
+
+  f32x4_t acc[WT][MB];
+#pragma unroll
+  for (int t = 0; t < WT; ++t)
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[t][b] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  // Every load has the same number of younger loads behind it when it is waited for, in the
+  // first chunks as in the later ones (the order of issue before the loop is the loop's), so
+  // the waits the compiler counts out leave the rest of the ring in flight.
+  bf16x8_t w[DEPTH][KC][WT], ar[UPW], zero;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) zero[e] = (bf16_t)0.0f;
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) {
+    const int s_w = chunk_start(d);
+#pragma unroll
+    for (int s = 0; s < KC; ++s)
+#pragma unroll
+      for (int t = 0; t < WT; ++t)
+        w[d][s][t] = ((const bf16x8_t*)(wbase[t] + (size_t)min(s_w + s, last_step) * wstep[t % NT]))[lane];
+  }
+  {
+    const int s_a = chunk_start(0);
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) ar[j] = *(const bf16x8_t*)(abase[j] + (min(s_a + apair[j], last_pair) << 5));
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) *(bf16x8_t*)(group_buf + awrite[j]) = ar[j];
+    const int s_a1 = chunk_start(1);
+#pragma unroll
+    for (int j = 0; j < UPW; ++j) ar[j] = *(const bf16x8_t*)(abase[j] + (min(s_a1 + apair[j], last_pair) << 5));
+  }
+
+  for (int c0 = 0; c0 < chunks; c0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int c = c0 + d;  // with an odd number of chunks and DEPTH 2 the last one is empty
+      __syncthreads();       // chunk c is staged, and nobody reads the other buffer any more
+      const unsigned char* cur = group_buf + (c & 1) * KC * SS + aread;
+      unsigned char* nxt = group_buf + ((c + 1) & 1) * KC * SS;
+      const int s_cur = chunk_start(c), s_w = chunk_start(c + DEPTH), s_a = chunk_start(c + 2);
+      const int n_live = g1 - s_cur;
+      // the activations of step s + 1 leave LDS while the products of step s run
+      bf16x8_t a[2][MB];
+#pragma unroll
+      for (int b = 0; b < MB; ++b) a[0][b] = *(const bf16x8_t*)(cur + b * BS);
+#pragma unroll
+      for (int s = 0; s < KC; ++s) {
+        if (s + 1 < KC) {
+#pragma unroll
+          for (int b = 0; b < MB; ++b) a[(s + 1) & 1][b] = *(const bf16x8_t*)(cur + (s + 1) * SS + b * BS);
+        }
+        // a step past the group's end counts as zeros: a select, because a branch round the
+        // products would make the accumulators leave their registers at every step
+        const bool live = s < n_live;
+#pragma unroll
+        for (int t = 0; t < WT; ++t) {
+          const bf16x8_t wt = live ? w[d][s][t] : zero;
+#pragma unroll
+          for (int b = 0; b < MB; ++b)
+            acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wt, a[s & 1][b], acc[t][b], 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < WT; ++t)
+          w[d][s][t] = ((const bf16x8_t*)(wbase[t] + (size_t)min(s_w + s, last_step) * wstep[t % NT]))[lane];
+      }
+      // the activations of chunk c + 1, asked for a chunk ago, go to the other buffer; those
+      // of chunk c + 2 are asked for
+#pragma unroll
+      for (int j = 0; j < UPW; ++j) *(bf16x8_t*)(nxt + awrite[j]) = ar[j];
+#pragma unroll
+      for (int j = 0; j < UPW; ++j)
+        ar[j] = *(const bf16x8_t*)(abase[j] + (min(s_a + apair[j], last_pair) << 5));
+    }
+  }
+
+  if (KW > 1) {  // the K groups' sums meet in group 0, added in group order
+    __syncthreads();
+    float* red = (float*)smem_raw;  // [KW - 1][NWV][WT][MB][4][64]
+    if (kg > 0) {
+#pragma unroll
+      for (int t = 0; t < WT; ++t)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            red[(((((kg - 1) * NWV + nw) * WT + t) * MB + b) * 4 + r) * 64 + lane] = acc[t][b][r];
+    }
+    __syncthreads();
+    if (kg > 0) return;
+    for (int g = 1; g < KW; ++g)
+#pragma unroll
+      for (int t = 0; t < WT; ++t)
+#pragma unroll
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            acc[t][b][r] += red[(((((g - 1) * NWV + nw) * WT + t) * MB + b) * 4 + r) * 64 + lane];
+  }
+
+  // acc[t][b][r]: output row 16 b + r16, column 16 (tile0 + t) + 4 quad + r: one vector store
+  C += (size_t)blockIdx.y * M * N;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    if (tile0 + t >= tile_hi) continue;
+    const int n = 16 * (tile0 + t) + 4 * quad;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const int m = 16 * b + r16;
+      if (m >= M) continue;
+      float o[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (GATED) {  // gate and up value rounded to bfloat16 first, as the unfused kernels see them
+          const float g = (float)(bf16_t)acc[t][b][r];
+          o[r] = g / (1.0f + expf(-g)) * (float)(bf16_t)acc[NT + t][b][r];
+        } else {
+          o[r] = acc[t][b][r];
+        }
+      }
+      store4(C + (size_t)m * N + n, o);
+    }
+  }
+}
+
+template <int MB, int KW, int NWV, int NT, int KC, int DEPTH, bool GATED>
+static int launch_mid(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K,
+                      hipStream_t stream, int k_parts) {
+  constexpr int WT = GATED ? 2 * NT : NT;
+  const int per_block = NWV * NT, tiles = N / 16;
+  // as many blocks as compute units where the tiles allow it, each with its even share
+  int blocks = tiles <= 256 / k_parts ? tiles : max(256 / k_parts, (tiles + per_block - 1) / per_block);
+  blocks = max(blocks, (tiles + per_block - 1) / per_block);
+  dim3 grid(blocks, k_parts), block(64 * KW * NWV);
+  const size_t stage = (size_t)KW * 2 * KC * (MB * 4 * (256 + 16) + 64);
+  const size_t meet = (size_t)(KW - 1) * NWV * WT * MB * 1024;
+  const size_t smem = stage > meet ? stage : meet;
+  QRT_CHECK(smem <= 160 * 1024, "gemm_bf16: the staging of this configuration needs %zu bytes of LDS", smem);
+#define GO(TO)                                                                                          \
+  do {                                                                                                  \
+    auto kernel = gemm_bf16_mid_kernel<MB, KW, NWV, NT, KC, DEPTH, GATED, TO>;                          \
+    static bool allowed = false; /* once per kernel: not inside a stream capture again and again */    \
+    if (smem > 64 * 1024 && !allowed) {                                                                 \
+      if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
+        return qrt_fail("gemm_bf16: cannot get %zu bytes of LDS", smem);                                \
+      allowed = true;                                                                                   \
+    }                                                                                                   \
+    kernel<<<grid, block, smem, stream>>>(a, w, (TO*)c, M, N, K);                                       \
+  } while (0)
+  if (out_dtype == QRT_BF16) GO(bf16_t);
+  else if (out_dtype == QRT_F32) GO(float);
+  else return qrt_fail("gemm_bf16: unknown output dtype %d", out_dtype);
+#undef GO
+  QRT_LAUNCH_CHECK("gemm_bf16_mid");
+  return 0;
+}
+
+// 17 to 64 rows on tile-major weights. Configurations from timing a dozen of them on the
+// shapes of the 4B model at 32 and 64 rows: two K groups of two waves with two tiles each where
+// the result is wanted whole; one group of three waves, a gate and an up tile each, for the
+// gated form; one group of three waves with two tiles each where K is cut over blocks.
+template <int MB>
+static int mid(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K, int gated,
+               hipStream_t st, int k_parts) {
+  if (gated) return launch_mid<MB, 1, 3, 1, 6, 2, true>(a, w, c, out_dtype, M, N, K, st, 1);
+  if (k_parts > 1) return launch_mid<MB, 1, 3, 2, 6, 1, false>(a, w, c, out_dtype, M, N, K, st, k_parts);
+  return launch_mid<MB, 2, 2, 2, 4, 2, false>(a, w, c, out_dtype, M, N, K, st, 1);
 }
 
 template <int MT, int NT>
@@ -293,7 +549,8 @@ extern "C" int qrt_gemm_bf16_variant(const void* a, const void* w, void* c, int 
 // gated = 0: C[M, N] = A W^T with W [N, K].
 // gated = 1: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A Wg^T) * (A Wu^T).
 // tiled = 1: W is stored tile-major, [rows / 16][K / 32][64 lanes][8]: lane q * 16 + i of tile
-// (r, s) holds W[16 r + i][32 s + 8 q .. + 7]; needs M <= 16, N % 16 == 0, K % 32 == 0.
+// (r, s) holds W[16 r + i][32 s + 8 q .. + 7]; needs M <= 64, N % 16 == 0, K % 32 == 0, and
+// K % 64 == 0 above 16 rows.
 // k_parts > 1 (tile-major, not gated, float32 out): K is cut into that many parts, each handled
 // by blocks of its own, and C is [k_parts, M, N]: planes to be added by the caller.
 extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K, int gated,
@@ -308,14 +565,21 @@ extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtyp
   const bf16_t* W = (const bf16_t*)w;
   const bool aligned = (K % 32 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
   if (tiled) {
-    QRT_CHECK(M <= 16 && N % 16 == 0 && aligned,
-              "gemm_bf16: tile-major weights need M <= 16, N %% 16 == 0, K %% 32 == 0 (M=%d N=%d K=%d)", M, N, K);
-    return gated ? skinny_tiled<true>(A, W, c, out_dtype, M, N, K, stream, 1)
-                 : skinny_tiled<false>(A, W, c, out_dtype, M, N, K, stream, k_parts);
+    QRT_CHECK(M <= 64 && N % 16 == 0 && aligned,
+              "gemm_bf16: tile-major weights need M <= 64, N %% 16 == 0, K %% 32 == 0 (M=%d N=%d K=%d)", M, N, K);
+    if (M <= 16)
+      return gated ? skinny_tiled<true>(A, W, c, out_dtype, M, N, K, stream, 1)
+                   : skinny_tiled<false>(A, W, c, out_dtype, M, N, K, stream, k_parts);
+    QRT_CHECK(K % 64 == 0 && N <= (1 << 20),
+              "gemm_bf16: 17 to 64 rows on tile-major weights need K %% 64 == 0 and N <= 2^20 (N=%d K=%d)", N, K);
+    if (M <= 32) return mid<2>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
+    if (M <= 48) return mid<3>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
+    return mid<4>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
   }
-  if (M <= 64 && aligned) return gated ? skinny<true>(A, W, c, out_dtype, M, N, K, stream)
+  if (M <= 16 && aligned) return gated ? skinny<true>(A, W, c, out_dtype, M, N, K, stream)
                                        : skinny<false>(A, W, c, out_dtype, M, N, K, stream);
-  QRT_CHECK(gated == 0, "gemm_bf16: the gated form needs M <= 64 and K a multiple of 32 (M=%d K=%d)", M, K);
+  QRT_CHECK(gated == 0, "gemm_bf16: the gated form needs K a multiple of 32, and M <= 16 or tile-major weights "
+            "(M=%d K=%d)", M, K);
   if (M <= 16) return launch<1, 2>(A, W, c, out_dtype, M, N, K, stream);
   if (M <= 32) return launch<2, 2>(A, W, c, out_dtype, M, N, K, stream);
   return launch<4, 4>(A, W, c, out_dtype, M, N, K, stream);

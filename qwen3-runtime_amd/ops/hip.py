@@ -130,8 +130,9 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> torch.Tensor:
 
 
 class HipOps:
-    # bfloat16 products with more rows than this go to the vendor BLAS
-    own_max_rows = 16
+    # bfloat16 products with more rows than this go to the vendor BLAS (up to 16 rows any weight
+    # will do; from 17 rows on the own kernel wants the tile-major copy and K a multiple of 64)
+    own_max_rows = 64
     # tiles of 16 rows per wave in the attention kernel for long portions (1, 2 or 4)
     prefill_row_tiles = 2
     # long portions: keys and values go through LDS, shared by the four waves of a block
@@ -148,7 +149,8 @@ class HipOps:
 
         Tile (r, s) of 16 rows x 32 columns becomes one contiguous KB in the order the MFMA's
         lanes read it, so a wave's load is eight whole cache lines instead of sixteen halves:
-        measured 13 to 28 % faster on the 4B model's shapes. Costs the matrix's size again."""
+        measured 13 to 28 % faster on the 4B model's shapes up to 16 rows; the kernel for 17 to
+        64 rows reads nothing else. Costs the matrix's size again."""
         if w.dtype != torch.bfloat16 or w.dim() != 2 or not w.is_cuda:
             return
         n, k = w.shape
@@ -226,18 +228,26 @@ class HipOps:
             return out if (out_f32 or x.dtype == torch.float32) else out.to(x.dtype)
         if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
             raise OpsError(f"linear: no product of {x.dtype} activations with {w.dtype} weights")
-        if m > self.own_max_rows:
-            # measured at the 4B shapes: from about 32 rows on the vendor library streams the
-            # weights faster than the few-row kernel; both accumulate in float32
+        tiled = self._tiled_copy(w)
+        if not self._own_kernel_takes(m, k, tiled):
+            # many rows: the vendor library; both accumulate in float32
             if out_f32:
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
             return torch.matmul(x, w.t())
         out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
-        tiled = self._tiled_copy(w)
         self._check(self.lib, self.lib.qrt_gemm_bf16(
             _ptr(x), _ptr(w if tiled is None else tiled), _ptr(out), F32 if out_f32 else BF16,
             c_int(m), c_int(n), c_int(k), c_int(0), c_int(0 if tiled is None else 1), c_int(1), _stream()))
         return out
+
+    def _own_kernel_takes(self, m: int, k: int, tiled) -> bool:
+        """Rows up to 16: the few-row kernel, on any weight layout. 17 to ``own_max_rows``: the
+        kernel that shares the activations through LDS, on the tile-major copy only (measured at
+        the 4B shapes, 32 and 64 rows: 28 to 32 % less time than the vendor library over the four
+        products of a layer). Without the copy, or beyond, the vendor library."""
+        if m <= min(16, self.own_max_rows):
+            return True
+        return m <= self.own_max_rows and tiled is not None and k % 64 == 0
 
     def linear_for_residual(self, x, w):
         """``linear(x, w)`` for a result that is only ever added to the residual stream.
@@ -247,8 +257,10 @@ class HipOps:
         per row tile, which fills the chip (160 row tiles for 256 compute units at the 4B size)."""
         m, k = x.shape
         n = w.shape[0]
-        tiled = self._tiled_copy(w) if (x.dtype == torch.bfloat16 and m <= self.own_max_rows) else None
-        parts = self.choose_k_parts(n, k) if tiled is not None else 1
+        tiled = self._tiled_copy(w) if x.dtype == torch.bfloat16 else None
+        if tiled is None or not self._own_kernel_takes(m, k, tiled):
+            return self.linear(x, w)
+        parts = self.choose_k_parts(n, k, m)
         if parts == 1:
             return self.linear(x, w)
         _need(x, "x", torch.bfloat16)
@@ -259,15 +271,21 @@ class HipOps:
         return out
 
     @staticmethod
-    def choose_k_parts(n: int, k: int) -> int:
-        """Cut K when there are fewer row tiles than about two per compute unit and K is long."""
+    def choose_k_parts(n: int, k: int, m: int = 1) -> int:
+        """Up to 16 rows: cut K when there are fewer row tiles than about two per compute unit
+        and K is long. 17 to 64 rows: a block takes up to six row tiles, so that they share the
+        activations, and K is cut until there are about as many blocks as compute units, each
+        part keeping 12 k-steps or more."""
         tiles = n // 16
-        if tiles >= 384 or k < 2048:
-            return 1
-        return 2 if k < 8192 else 4
+        if m <= 16:
+            if tiles >= 384 or k < 2048:
+                return 1
+            return 2 if k < 8192 else 4
+        blocks = (tiles + 5) // 6
+        return max(1, min(8, 256 // blocks, (k // 32) // 12))
 
     # rows up to which the gated activation is fused into the product before it
-    fused_gate_max_rows = 16
+    fused_gate_max_rows = 64
 
     def gated_linear(self, x, w_gate_up):
         """``swiglu(linear(x, w_gate_up))`` with ``w_gate_up`` [2I, K], gate rows first. With few
@@ -281,12 +299,13 @@ class HipOps:
                 and k % 32 == 0):
             _need(x, "x")
             _need(w_gate_up, "weight")
-            out = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
             tiled = self._tiled_copy(w_gate_up) if (two_i // 2) % 16 == 0 else None
-            self._check(self.lib, self.lib.qrt_gemm_bf16(
-                _ptr(x), _ptr(w_gate_up if tiled is None else tiled), _ptr(out), BF16, c_int(m),
-                c_int(two_i // 2), c_int(k), c_int(1), c_int(0 if tiled is None else 1), c_int(1), _stream()))
-            return out
+            if self._own_kernel_takes(m, k, tiled):
+                out = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
+                self._check(self.lib, self.lib.qrt_gemm_bf16(
+                    _ptr(x), _ptr(w_gate_up if tiled is None else tiled), _ptr(out), BF16, c_int(m),
+                    c_int(two_i // 2), c_int(k), c_int(1), c_int(0 if tiled is None else 1), c_int(1), _stream()))
+                return out
         return self.swiglu(self.linear(x, w_gate_up))
 
     # ---- q/k norm, rotation, cache write ----------------------------------------

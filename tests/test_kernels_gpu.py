@@ -138,14 +138,19 @@ def test_gated_linear(ops, m, i, k, monkeypatch):
         close(got, want, tol, tol)
 
 
-@pytest.mark.parametrize("own_max_rows", [16, 1 << 30])
-@pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 40, 64])
-@pytest.mark.parametrize("n,k", [(6144, 2560), (2560, 4096), (1000, 9728), (272, 96)])
-def test_gemm_bf16_few_rows_at_model_sizes(ops, m, n, k, own_max_rows, monkeypatch):
-    """Above ``own_max_rows`` rows the vendor library takes over; the library's own kernels for up
-    to 64 rows stay correct behind it."""
-    monkeypatch.setattr(ops, "own_max_rows", own_max_rows)
+@pytest.mark.parametrize("prepared", [False, True])
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 40, 64, 65])
+@pytest.mark.parametrize("n,k", [(6144, 2560), (2560, 4096), (1008, 9728), (272, 96), (272, 192)])
+def test_gemm_bf16_few_rows_at_model_sizes(m, n, k, prepared):
+    """Up to 16 rows the few-row kernel, on either weight layout; 17 to 64 rows the kernel that
+    shares the activations through LDS if there is a tile-major copy and K is a multiple of 64;
+    otherwise, and beyond, the vendor library. All of them against a float64 product."""
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    ops = HipOps()
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.02)
+    if prepared:
+        ops.prepare_weight(w)
     want = x.double() @ w.double().T
     got = ops.linear(x, w, out_f32=True)
     assert got.dtype == torch.float32
@@ -153,9 +158,10 @@ def test_gemm_bf16_few_rows_at_model_sizes(ops, m, n, k, own_max_rows, monkeypat
     close(ops.linear(x, w), want, 3e-2, 3e-2)
 
 
-@pytest.mark.parametrize("m", [1, 3, 8, 16])
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 31, 33, 48, 64])
 @pytest.mark.parametrize("n,k,gated", [(6144, 2560, False), (2560, 4096, False), (608, 9728, False), (64, 64, False),
-                                       (9728, 2560, True), (48, 96, True), (151936, 256, False)])
+                                       (9728, 2560, True), (48, 96, True), (151936, 256, False), (80, 128, True),
+                                       (4112, 640, True), (16, 64, False)])
 def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
     """A prepared weight (tile-major copy) gives the products of the plain one: both agree with a
     float64 product (the two may add partial sums in different orders)."""
@@ -175,8 +181,8 @@ def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
         close(prepared.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
         close(plain.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
         close(prepared.linear(x, w), want, 3e-2, 3e-2)
-    # more rows than the few-row kernel takes: the copy is not used, the result is the library's
-    big = rnd(40, k, dtype=torch.bfloat16, seed=3)
+    # more rows than the own kernels take: the copy is not used, the result is the library's
+    big = rnd(100, k, dtype=torch.bfloat16, seed=3)
     if not gated:
         assert torch.equal(prepared.linear(big, w), plain.linear(big, w))
     # sizes that cannot be tiled are left alone
@@ -185,8 +191,8 @@ def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
     assert prepared._tiled_copy(odd) is None
 
 
-@pytest.mark.parametrize("m", [1, 8, 16, 40])
-@pytest.mark.parametrize("n,k", [(2560, 4096), (2560, 9728), (96, 2048), (6144, 2560), (64, 64)])
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 70])
+@pytest.mark.parametrize("n,k", [(2560, 4096), (2560, 9728), (96, 2048), (6144, 2560), (64, 64), (4096, 12288)])
 def test_product_for_the_residual_may_come_in_planes(m, n, k):
     """linear_for_residual's planes sum to the product, and add_rmsnorm adds them like one delta."""
     from qwen3_runtime_amd.ops.hip import HipOps
@@ -197,8 +203,8 @@ def test_product_for_the_residual_may_come_in_planes(m, n, k):
     ops.prepare_weight(w)
     want = x.double() @ w.double().T
     got = ops.linear_for_residual(x, w)
-    if m <= 16 and n // 16 < 384 and k >= 2048:
-        assert got.dim() == 3 and got.shape[0] == ops.choose_k_parts(n, k) > 1 and got.dtype == torch.float32
+    if m <= 64 and ops.choose_k_parts(n, k, m) > 1:
+        assert got.dim() == 3 and got.shape[0] == ops.choose_k_parts(n, k, m) and got.dtype == torch.float32
         close(got.sum(0), want, 2e-3, 2e-3)
     else:
         assert got.dim() == 2
