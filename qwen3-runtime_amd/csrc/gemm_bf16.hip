@@ -506,6 +506,8 @@ static int mid(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, 
                hipStream_t st, int k_parts) {
   if (gated) return launch_mid<MB, 1, 3, 1, 6, 2, true>(a, w, c, out_dtype, M, N, K, st, 1);
   if (k_parts > 1) return launch_mid<MB, 1, 3, 2, 6, 1, false>(a, w, c, out_dtype, M, N, K, st, k_parts);
+  // very many tiles (the vocabulary head): eight tiles share the staged activations
+  if (N >= 32768) return launch_mid<MB, 1, 4, 2, 8, 1, false>(a, w, c, out_dtype, M, N, K, st, 1);
   return launch_mid<MB, 2, 2, 2, 4, 2, false>(a, w, c, out_dtype, M, N, K, st, 1);
 }
 
