@@ -86,16 +86,20 @@ constexpr int DB = D / 16;           // 16-wide blocks of the head dimension
 template <bool P2> __device__ __forceinline__ int page_div(int x, int ps, int shift) { return P2 ? x >> shift : x / ps; }
 template <bool P2> __device__ __forceinline__ int page_mod(int x, int ps) { return P2 ? x & (ps - 1) : x % ps; }
 
+// The larger of two, a NaN if either is one (IEEE 754-2019 maximum): one instruction, where
+// fmaxf first quiets every operand whose origin the compiler cannot see (three for one).
+__device__ __forceinline__ float max2(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+
 // max over the four lanes that hold one row (lane, lane ^ 16, lane ^ 32, lane ^ 48): two swaps of
 // register halves between rows of 16 lanes, no LDS traffic and no address arithmetic
 __device__ __forceinline__ float row_max4(float x) {
   typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
   const unsigned int u = __float_as_uint(x);
   const u32x2_t a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const float y = max2(__uint_as_float(a[0]), __uint_as_float(a[1]));
   const unsigned int v = __float_as_uint(y);
   const u32x2_t b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+  return max2(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
 __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t* vv, bool masked, int base,
@@ -114,9 +118,9 @@ __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t*
   }
   float mx = -INFINITY;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) mx = fmaxf(mx, s[e]);
+  for (int e = 0; e < 8; ++e) mx = max2(mx, s[e]);
   mx = row_max4(mx);
-  const float m_new = fmaxf(m, mx * scale_log2);
+  const float m_new = max2(m, mx * scale_log2);
   const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
   // v_exp_f32 directly: results below the normal range may flush to zero, which is what they are worth here
   const float corr = __builtin_amdgcn_exp2f(m - m_use);
@@ -171,9 +175,9 @@ __device__ __forceinline__ void tiles_update(const f32x4_t (*sc)[2], const bf16x
   for (int t = 0; t < RT; ++t) {
     float mx = -INFINITY;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, s[t][e]);
+    for (int e = 0; e < 8; ++e) mx = max2(mx, s[t][e]);
     mx = row_max4(mx);
-    const float m_new = fmaxf(m[t], mx * scale_log2);
+    const float m_new = max2(m[t], mx * scale_log2);
     m_use[t] = m_new == -INFINITY ? 0.f : m_new;
     corr[t] = __builtin_amdgcn_exp2f(m[t] - m_use[t]);
     m[t] = m_new;
