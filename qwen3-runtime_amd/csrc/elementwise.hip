@@ -159,7 +159,7 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
   const bool vec4 = hidden % 4 == 0 && (uintptr_t)residual % 16 == 0 && (uintptr_t)weight % 16 == 0 &&
                     (uintptr_t)out % 16 == 0 && (!delta || (uintptr_t)delta % 16 == 0) && plane_stride % 4 == 0;
   // planes known to the compiler (0: no delta) where the count is a usual one
-  const int pl = !delta ? 0 : (planes == 1 || planes == 2 || planes == 4) ? planes : -1;
+  const int pl = !delta ? 0 : (planes == 1 || planes == 2 || planes == 4 || planes == 8) ? planes : -1;
 #define GO(TD, TO, VEC, KEEP, PL)                                                                               \
   add_rmsnorm_kernel<TD, TO, VEC, KEEP, PL><<<grid, block, 0, stream>>>(residual, (const TD*)delta, weight,     \
                                                                         rows, (TO*)out, hidden, eps, planes,    \
@@ -171,6 +171,7 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
     else if (pl == 1) GO(TD, TO, 4, 4, 1);                                                                      \
     else if (pl == 2) GO(TD, TO, 4, 4, 2);                                                                      \
     else if (pl == 4) GO(TD, TO, 4, 4, 4);                                                                      \
+    else if (pl == 8) GO(TD, TO, 4, 4, 8);                                                                      \
     else GO(TD, TO, 4, 4, -1);                                                                                  \
   } while (0)
   if (delta_dtype == QRT_F32 && out_dtype == QRT_F32) LAUNCH(float, float);
