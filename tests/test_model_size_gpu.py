@@ -79,6 +79,38 @@ def test_model_sized_layers_match_plain(sized_folders, plain_results, name, dtyp
         check_rounding_noise(got, want)
 
 
+@pytest.mark.parametrize("live", [20, 40, 64])
+def test_many_requests_decode_together_at_model_sizes(sized_folders, live):
+    """17 to 64 requests decoding in one step at the 4B layer sizes: the products with that many
+    rows (own kernel on tile-major weights: whole result, gated, K cut into planes), decode
+    attention over many sequences. Prompts in three steps, then six steps with a token of every
+    request, against the plain implementation of each request alone."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg, folder = sized_folders["qwen3_4b"]
+    lengths = [9 + (5 * i) % 23 for i in range(live)]
+    reqs = traces.make_requests(cfg.vocab_size, lengths, seed=30 + live)
+    rids = list(reqs)
+    steps, decode = [], 6
+    for lo in range(0, live, (live + 2) // 3):
+        part = rids[lo: lo + (live + 2) // 3]
+        steps.append({"entries": [{"id": r, "tokens": reqs[r][:-decode], "want": [len(reqs[r]) - decode - 1]}
+                                  for r in part], "end": []})
+    for d in range(decode, 0, -1):
+        steps.append({"entries": [{"id": r, "tokens": reqs[r][len(reqs[r]) - d: len(reqs[r]) - d + 1], "want": [0]}
+                                  for r in rids], "end": rids if d == 1 else []})
+    steps = traces._number(steps)
+    want_all = traces.plain_logits(folder, reqs)
+    engine_cfg = EngineConfig(page_size=16, num_pages=live * 3, max_num_seqs=live, max_num_batched_tokens=1024,
+                              dtype="bfloat16", device="cuda:0", hip_graph=False)
+    loaded = load(folder, engine_cfg)
+    assert loaded.runner.ops._tiled, "the weights have tile-major copies: the own kernels run"
+    got = traces.replay(loaded, steps)
+    assert len(got) == live * (decode + 1)
+    check_rounding_noise(got, {k: want_all[k] for k in got})
+
+
 def test_model_sized_decode_graph_equals_eager(sized_folders):
     """Greedy tokens of three requests at the 4B layer sizes: replayed HIP graphs give the tokens
     of eager steps."""
