@@ -86,6 +86,14 @@ constexpr int DB = D / 16;           // 16-wide blocks of the head dimension
 template <bool P2> __device__ __forceinline__ int page_div(int x, int ps, int shift) { return P2 ? x >> shift : x / ps; }
 template <bool P2> __device__ __forceinline__ int page_mod(int x, int ps) { return P2 ? x & (ps - 1) : x % ps; }
 
+// ``v`` if ``keep``, else zeros: four 32-bit selects (element by element it was sixteen
+// instructions with the shifts and packs around them)
+__device__ __forceinline__ bf16x8_t keep_or_zero(bf16x8_t v, bool keep) {
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+  const u32x4_t bits = __builtin_bit_cast(u32x4_t, v);
+  return __builtin_bit_cast(bf16x8_t, keep ? bits : (u32x4_t){0u, 0u, 0u, 0u});
+}
+
 // The larger of two, a NaN if either is one (IEEE 754-2019 maximum): one instruction, where
 // fmaxf first quiets every operand whose origin the compiler cannot see (three for one).
 __device__ __forceinline__ float max2(float a, float b) { return __builtin_elementwise_maximum(a, b); }
@@ -148,24 +156,23 @@ __device__ __forceinline__ void tile_update(const f32x4_t sc[2], const bf16x8_t*
 // on each other, and written side by side in one stretch of code without branches between them
 // the exponentials of one tile can issue while the matrix pipe works on another's products.
 template <int RT>
-__device__ __forceinline__ void tiles_update(const f32x4_t (*sc)[2], const bf16x8_t* vv, const bool* whole, int base,
+__device__ __forceinline__ void tiles_update(const f32x4_t (*sc)[2], const bf16x8_t* vv, unsigned whole, int base,
                                              int quad, const bool* row_valid, const int* qpos, int window,
                                              float scale_log2, float* m, float* l, f32x4_t (*o)[DB]) {
+  // whole: bit t says that every row of tile t sees all 32 keys (one scalar for the wave: an
+  // array of flags went through vector registers, a dozen instructions per block of keys)
   float s[RT][8];
-  bool any_masked = false;
 #pragma unroll
-  for (int t = 0; t < RT; ++t) {
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
     for (int e = 0; e < 8; ++e) s[t][e] = sc[t][e >> 2][e & 3];
-    any_masked |= !whole[t];
-  }
-  if (any_masked) {  // the same for the whole wave
+  if (whole != (1u << RT) - 1) {  // the same for the whole wave
 #pragma unroll
     for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = base + 8 * quad + e;
-        const bool vis = whole[t] || (row_valid[t] && key <= qpos[t] && (window == 0 || key > qpos[t] - window));
+        const bool vis = ((whole >> t) & 1) || (row_valid[t] && key <= qpos[t] && (window == 0 || key > qpos[t] - window));
         s[t][e] = vis ? s[t][e] : -INFINITY;
       }
   }
@@ -331,9 +338,7 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
       if (base < lo || base + 31 > pos_max) {  // the same for the whole wave
         const bool seen = kv0 <= pos_max && kv0 + 7 >= lo;
 #pragma unroll
-        for (int i = 0; i < DB; ++i)
-#pragma unroll
-          for (int e = 0; e < 8; ++e) blk.v[i][e] = seen ? blk.v[i][e] : (bf16_t)0.0f;
+        for (int i = 0; i < DB; ++i) blk.v[i] = keep_or_zero(blk.v[i], seen);
       }
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
@@ -513,10 +518,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
         const int kl = c / (D / 8), part = c - kl * (D / 8);
         const int row = 16 * (kl >> 2) + (w8 >> 1) + (kl & 3);
         *(bf16x8_t*)(kb + row * KROW + 8 * part) = kpiece[i];
-        bf16x8_t v = vpiece[i];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = seen ? v[e] : (bf16_t)0.0f;
-        *(bf16x8_t*)(vb + c * VROW + w8) = v;
+        *(bf16x8_t*)(vb + c * VROW + w8) = keep_or_zero(vpiece[i], seen);
       }
     }
   };
@@ -556,7 +558,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
       for (int i = 0; i < DB; ++i) vv[i] = *(const bf16x8_t*)(vb + (16 * i + r16) * VROW + 8 * quad);
 
       f32x4_t sc[RT][2];
-      bool whole[RT];
+      unsigned whole = 0;
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
 #pragma unroll
@@ -569,7 +571,8 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
           sc[t][s2] = acc;
         }
         // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
-        whole[t] = base + 31 <= tile_pos_min[t] && (a.window == 0 || base > tile_pos_max[t] - a.window);
+        const int sees_all = (base + 31 <= tile_pos_min[t]) & ((a.window == 0) | (base > tile_pos_max[t] - a.window));
+        whole |= (unsigned)sees_all << t;
       }
       tiles_update<RT>(sc, vv, whole, base, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
     }
@@ -661,9 +664,7 @@ __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg
     const int kv0 = base + 8 * quad;
     const bool seen = kv0 <= pos_max && kv0 + 7 >= lo;
 #pragma unroll
-    for (int i = 0; i < DB; ++i)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) blk.v[i][e] = seen ? blk.v[i][e] : (bf16_t)0.0f;
+    for (int i = 0; i < DB; ++i) blk.v[i] = keep_or_zero(blk.v[i], seen);
   }
   tile_update(s, blk.v, !whole, base, quad, row_valid, qpos, window, scale_log2, m, l, o);
 }
