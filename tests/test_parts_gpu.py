@@ -141,7 +141,7 @@ def test_attention_mixer_alone(dtype, nq, nkv, d, h, theta, eps):
 # A toy architecture, registered from here.
 # ------------------------------------------------------------------------------------------------
 def register_toy():
-    from qwen3_runtime_amd.parts.base import Mixer, PositionEncoding
+    from qwen3_runtime_amd.parts.base import FeedForward, Mixer, PositionEncoding
     from qwen3_runtime_amd.parts.plan import CacheSpec, LayerSpec, ModelPlan, PartSpec, RunStep, TensorDecl
     from qwen3_runtime_amd.registry import register_architecture, register_part
 
@@ -186,6 +186,44 @@ def register_toy():
             f = (1.0 + self.rate * ctx.positions.float())[:, None, None]
             return (q.float() * f).to(q.dtype), (k.float() * f).to(k.dtype)
 
+    @register_part("feed_forward", "toy_routed")
+    class RoutedFeedForward(FeedForward):
+        """Experts with a router: p = softmax(scale * router x) in float32, an expert's weight is
+        max(p - floor, 0) over the sum of these, and an expert runs only over the tokens that give
+        it a weight (the weights are continuous in x, so rounding cannot flip a choice)."""
+
+        def __init__(self, hidden_size, intermediate_size, experts, scale, floor, tensors=None):
+            super().__init__(tensors)
+            self.h, self.i, self.e, self.scale, self.floor = hidden_size, intermediate_size, experts, scale, floor
+            self.router, self.gate_up, self.down = None, [], []
+
+        def tensor_decls(self):
+            decls = [TensorDecl(self._name("router"), (self.e, self.h))]
+            for e in range(self.e):
+                decls += [TensorDecl(f"{self._name('expert')}.{e}.gate", (self.i, self.h)),
+                          TensorDecl(f"{self._name('expert')}.{e}.up", (self.i, self.h)),
+                          TensorDecl(f"{self._name('expert')}.{e}.down", (self.h, self.i))]
+            return decls
+
+        def load(self, fetch):
+            self.router = fetch.matrix(self._name("router"), linear=False)
+            for e in range(self.e):
+                base = f"{self._name('expert')}.{e}"
+                self.gate_up.append(fetch.fused([f"{base}.gate", f"{base}.up"], dim=0))
+                self.down.append(fetch.matrix(f"{base}.down"))
+
+        def forward(self, ctx, x):
+            p = torch.softmax(self.scale * (x.float() @ self.router.float().T), dim=-1)
+            w = (p - self.floor).clamp_min(0)
+            w = w / w.sum(-1, keepdim=True)
+            out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+            for e in range(self.e):
+                rows = (w[:, e] > 0).nonzero().flatten()
+                if rows.numel():
+                    act = ctx.ops.gated_linear(x.index_select(0, rows).contiguous(), self.gate_up[e])
+                    out.index_add_(0, rows, ctx.ops.linear(act, self.down[e], out_f32=True) * w[rows, e, None])
+            return out.to(x.dtype)
+
     def read_config(raw):
         return dict(raw)
 
@@ -205,14 +243,19 @@ def register_toy():
             return PartSpec("swiglu", {"hidden_size": h, "intermediate_size": c["intermediate_size"]},
                             {k: f"toy.{i}.ff.{k}" for k in ("gate", "up", "down")})
 
-        def layer(i, mixer):
-            return LayerSpec(PartSpec("pre_norm"), mixer, ff(i),
+        def routed(i):
+            return PartSpec("toy_routed", {"hidden_size": h, "intermediate_size": c["expert_size"], "experts": c["experts"],
+                                           "scale": c["router_scale"], "floor": c["router_floor"]},
+                            {"router": f"toy.{i}.router", "expert": f"toy.{i}.expert"})
+
+        def layer(i, mixer, feed_forward=None):
+            return LayerSpec(PartSpec("pre_norm"), mixer, feed_forward or ff(i),
                              {"input": norm(f"toy.{i}.norm_in"), "post_mixer": norm(f"toy.{i}.norm_post")})
 
         rope = PartSpec("rope_neox", {"head_dim": d, "theta": c["theta"]})
         layers = [
             layer(0, attn(0, 4, 2, rope)),
-            layer(1, PartSpec("toy_ema", {"hidden_size": h, "decay": 0.7}, {"gain": "toy.1.gain"})),
+            layer(1, PartSpec("toy_ema", {"hidden_size": h, "decay": 0.7}, {"gain": "toy.1.gain"}), routed(1)),
             layer(2, attn(2, 2, 1, PartSpec("toy_scale", {"rate": 0.02}), window=c["window"])),
         ]
         kv = lambda heads, window=None: CacheSpec("paged_kv", heads=heads, head_dim=d, window=window)
@@ -227,7 +270,8 @@ def register_toy():
 
 
 TOY = {"architectures": ["ToyMixedForCausalLM"], "vocab_size": 200, "hidden_size": 48, "head_dim": 16,
-       "intermediate_size": 80, "eps": 1e-5, "theta": 5000.0, "window": 11, "max_positions": 512}
+       "intermediate_size": 80, "eps": 1e-5, "theta": 5000.0, "window": 11, "max_positions": 512,
+       "experts": 3, "expert_size": 48, "router_scale": 30.0, "router_floor": 0.3}
 
 
 def toy_plain(folder, ids):
@@ -263,14 +307,29 @@ def toy_plain(folder, ids):
             out.append(w["toy.1.gain"] * state)
         return torch.stack(out)
 
-    def block(i, x, mix):
+    def routed(i, n):
+        p = torch.softmax(c["router_scale"] * (n @ w[f"toy.{i}.router"].T), dim=-1)
+        wt = (p - c["router_floor"]).clamp_min(0)
+        wt = wt / wt.sum(-1, keepdim=True)
+        out = torch.zeros_like(n)
+        for e in range(c["experts"]):
+            ffw = {f"f.{k}_proj.weight": w[f"toy.{i}.expert.{e}.{k}"] for k in ("gate", "up", "down")}
+            out = out + wt[:, e, None] * P.feed_forward(n, ffw, "f")
+        if t >= 30:  # the routing routes: every expert is left out by some tokens and taken by others
+            taken = (wt > 0).sum(0)
+            assert bool(((taken > 0) & (taken < t)).all()), taken
+        return out
+
+    def block(i, x, mix, routing=False):
         x = x + mix(P.rms_norm(x, w[f"toy.{i}.norm_in"], c["eps"]))
         n = P.rms_norm(x, w[f"toy.{i}.norm_post"], c["eps"])
+        if routing:
+            return x + routed(i, n)
         ffw = {f"f.{k}_proj.weight": w[f"toy.{i}.ff.{k}"] for k in ("gate", "up", "down")}
         return x + P.feed_forward(n, ffw, "f")
 
     x = block(0, x, lambda n: attn(0, 4, 2, n, False, None))
-    x = block(1, x, ema)
+    x = block(1, x, ema, routing=True)
     x = block(2, x, lambda n: attn(2, 2, 1, n, True, c["window"]))
     x = block(0, x, lambda n: attn(0, 4, 2, n, False, None))
     x = block(2, x, lambda n: attn(2, 2, 1, n, True, c["window"], reuse=True))
@@ -288,6 +347,7 @@ def toy_folder(tmp_path_factory):
     unregister_architecture("ToyMixedForCausalLM")
     unregister_part("mixer", "toy_ema")
     unregister_part("position", "toy_scale")
+    unregister_part("feed_forward", "toy_routed")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
