@@ -504,11 +504,17 @@ static int launch_mid(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, 
 template <int MB>
 static int mid(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K, int gated,
                hipStream_t st, int k_parts) {
-  if (gated) return launch_mid<MB, 1, 3, 1, 6, 2, true>(a, w, c, out_dtype, M, N, K, st, 1);
+  constexpr int DEPTH = MB <= 4 ? 2 : 1;  // more rows: more registers for activations, fewer for the weights' ring
+  if (gated) return launch_mid<MB, 1, 3, 1, 6, DEPTH, true>(a, w, c, out_dtype, M, N, K, st, 1);
   if (k_parts > 1) return launch_mid<MB, 1, 3, 2, 6, 1, false>(a, w, c, out_dtype, M, N, K, st, k_parts);
-  // very many tiles (the vocabulary head): eight tiles share the staged activations
-  if (N >= 32768) return launch_mid<MB, 1, 4, 2, 8, 1, false>(a, w, c, out_dtype, M, N, K, st, 1);
-  return launch_mid<MB, 2, 2, 2, 4, 2, false>(a, w, c, out_dtype, M, N, K, st, 1);
+  // The whole result of an ungated product: up to 64 rows only. Beyond, every block would have to
+  // fetch more activations than weights, and the vendor library was measured to be faster.
+  if constexpr (MB <= 4) {
+    // very many tiles (the vocabulary head): eight tiles share the staged activations
+    if (N >= 32768) return launch_mid<MB, 1, 4, 2, 8, 1, false>(a, w, c, out_dtype, M, N, K, st, 1);
+    return launch_mid<MB, 2, 2, 2, 4, 2, false>(a, w, c, out_dtype, M, N, K, st, 1);
+  }
+  return qrt_fail("gemm_bf16: above 64 rows only the gated form and products cut along K run on tile-major weights (M=%d)", M);
 }
 
 template <int MT, int NT>
@@ -551,8 +557,8 @@ extern "C" int qrt_gemm_bf16_variant(const void* a, const void* w, void* c, int 
 // gated = 0: C[M, N] = A W^T with W [N, K].
 // gated = 1: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A Wg^T) * (A Wu^T).
 // tiled = 1: W is stored tile-major, [rows / 16][K / 32][64 lanes][8]: lane q * 16 + i of tile
-// (r, s) holds W[16 r + i][32 s + 8 q .. + 7]; needs M <= 64, N % 16 == 0, K % 32 == 0, and
-// K % 64 == 0 above 16 rows.
+// (r, s) holds W[16 r + i][32 s + 8 q .. + 7]; needs N % 16 == 0, K % 32 == 0, K % 64 == 0 above 16
+// rows, and M <= 64 (M <= 128 for the gated form and for K parts).
 // k_parts > 1 (tile-major, not gated, float32 out): K is cut into that many parts, each handled
 // by blocks of its own, and C is [k_parts, M, N]: planes to be added by the caller.
 extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K, int gated,
@@ -567,16 +573,18 @@ extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtyp
   const bf16_t* W = (const bf16_t*)w;
   const bool aligned = (K % 32 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
   if (tiled) {
-    QRT_CHECK(M <= 64 && N % 16 == 0 && aligned,
-              "gemm_bf16: tile-major weights need M <= 64, N %% 16 == 0, K %% 32 == 0 (M=%d N=%d K=%d)", M, N, K);
+    QRT_CHECK(M <= 128 && N % 16 == 0 && aligned,
+              "gemm_bf16: tile-major weights need M <= 128, N %% 16 == 0, K %% 32 == 0 (M=%d N=%d K=%d)", M, N, K);
     if (M <= 16)
       return gated ? skinny_tiled<true>(A, W, c, out_dtype, M, N, K, stream, 1)
                    : skinny_tiled<false>(A, W, c, out_dtype, M, N, K, stream, k_parts);
     QRT_CHECK(K % 64 == 0 && N <= (1 << 20),
-              "gemm_bf16: 17 to 64 rows on tile-major weights need K %% 64 == 0 and N <= 2^20 (N=%d K=%d)", N, K);
+              "gemm_bf16: 17 to 128 rows on tile-major weights need K %% 64 == 0 and N <= 2^20 (N=%d K=%d)", N, K);
     if (M <= 32) return mid<2>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
     if (M <= 48) return mid<3>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
-    return mid<4>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
+    if (M <= 64) return mid<4>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
+    if (M <= 96) return mid<6>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
+    return mid<8>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
   }
   if (M <= 16 && aligned) return gated ? skinny<true>(A, W, c, out_dtype, M, N, K, stream)
                                        : skinny<false>(A, W, c, out_dtype, M, N, K, stream);

@@ -113,7 +113,16 @@ def _addr(t: torch.Tensor | None):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream() -> c_void_p:
+    """torch's current stream on the current device. The two calls behind the public
+    ``torch.cuda.current_stream()`` are used directly where this torch has them: the public one
+    builds a Stream object and cost 9 us a launch, a quarter of a short prompt step's host time."""
+    if _raw_stream is not None and _raw_device is not None:
+        return c_void_p(_raw_stream(_raw_device()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
@@ -133,6 +142,9 @@ class HipOps:
     # bfloat16 products with more rows than this go to the vendor BLAS (up to 16 rows any weight
     # will do; from 17 rows on the own kernel wants the tile-major copy and K a multiple of 64)
     own_max_rows = 64
+    # the same for the two forms in which a block fetches fewer activations than weights: the
+    # gated product, and the product cut along K whose planes the residual's norm adds
+    own_max_rows_shared = 128
     # tiles of 16 rows per wave in the attention kernel for long portions (1, 2 or 4)
     prefill_row_tiles = 2
     # long portions: keys and values go through LDS, shared by the four waves of a block
@@ -229,7 +241,7 @@ class HipOps:
         if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
             raise OpsError(f"linear: no product of {x.dtype} activations with {w.dtype} weights")
         tiled = self._tiled_copy(w)
-        if not self._own_kernel_takes(m, k, tiled):
+        if not self._own_kernel_takes(m, k, tiled, self.own_max_rows):
             # many rows: the vendor library; both accumulate in float32
             if out_f32:
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
@@ -240,14 +252,16 @@ class HipOps:
             c_int(m), c_int(n), c_int(k), c_int(0), c_int(0 if tiled is None else 1), c_int(1), _stream()))
         return out
 
-    def _own_kernel_takes(self, m: int, k: int, tiled) -> bool:
-        """Rows up to 16: the few-row kernel, on any weight layout. 17 to ``own_max_rows``: the
+    @staticmethod
+    def _own_kernel_takes(m: int, k: int, tiled, max_rows: int) -> bool:
+        """Rows up to 16: the few-row kernel, on any weight layout. 17 to ``max_rows``: the
         kernel that shares the activations through LDS, on the tile-major copy only (measured at
         the 4B shapes, 32 and 64 rows: 28 to 32 % less time than the vendor library over the four
-        products of a layer). Without the copy, or beyond, the vendor library."""
-        if m <= min(16, self.own_max_rows):
+        products of a layer; at 128 rows the gated product and the products cut along K take 71
+        us against the library's 116). Without the copy, or beyond, the vendor library."""
+        if m <= min(16, max_rows):
             return True
-        return m <= self.own_max_rows and tiled is not None and k % 64 == 0
+        return m <= max_rows and tiled is not None and k % 64 == 0
 
     def linear_for_residual(self, x, w):
         """``linear(x, w)`` for a result that is only ever added to the residual stream.
@@ -258,7 +272,7 @@ class HipOps:
         m, k = x.shape
         n = w.shape[0]
         tiled = self._tiled_copy(w) if x.dtype == torch.bfloat16 else None
-        if tiled is None or not self._own_kernel_takes(m, k, tiled):
+        if tiled is None or not self._own_kernel_takes(m, k, tiled, self.own_max_rows_shared):
             return self.linear(x, w)
         parts = self.choose_k_parts(n, k, m)
         if parts == 1:
@@ -273,7 +287,7 @@ class HipOps:
     @staticmethod
     def choose_k_parts(n: int, k: int, m: int = 1) -> int:
         """Up to 16 rows: cut K when there are fewer row tiles than about two per compute unit
-        and K is long. 17 to 64 rows: a block takes up to six row tiles, so that they share the
+        and K is long. 17 to 128 rows: a block takes up to six row tiles, so that they share the
         activations, and K is cut until there are about as many blocks as compute units, each
         part keeping 12 k-steps or more."""
         tiles = n // 16
@@ -285,7 +299,7 @@ class HipOps:
         return max(1, min(8, 256 // blocks, (k // 32) // 12))
 
     # rows up to which the gated activation is fused into the product before it
-    fused_gate_max_rows = 64
+    fused_gate_max_rows = 128
 
     def gated_linear(self, x, w_gate_up):
         """``swiglu(linear(x, w_gate_up))`` with ``w_gate_up`` [2I, K], gate rows first. With few
@@ -300,7 +314,7 @@ class HipOps:
             _need(x, "x")
             _need(w_gate_up, "weight")
             tiled = self._tiled_copy(w_gate_up) if (two_i // 2) % 16 == 0 else None
-            if self._own_kernel_takes(m, k, tiled):
+            if self._own_kernel_takes(m, k, tiled, self.fused_gate_max_rows):
                 out = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
                 self._check(self.lib, self.lib.qrt_gemm_bf16(
                     _ptr(x), _ptr(w_gate_up if tiled is None else tiled), _ptr(out), BF16, c_int(m),

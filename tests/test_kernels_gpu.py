@@ -158,7 +158,7 @@ def test_gemm_bf16_few_rows_at_model_sizes(m, n, k, prepared):
     close(ops.linear(x, w), want, 3e-2, 3e-2)
 
 
-@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 31, 33, 48, 64])
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 31, 33, 48, 64, 65, 96, 128])
 @pytest.mark.parametrize("n,k,gated", [(6144, 2560, False), (2560, 4096, False), (608, 9728, False), (64, 64, False),
                                        (9728, 2560, True), (48, 96, True), (151936, 256, False), (80, 128, True),
                                        (4112, 640, True), (16, 64, False)])
@@ -182,7 +182,7 @@ def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
         close(plain.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
         close(prepared.linear(x, w), want, 3e-2, 3e-2)
     # more rows than the own kernels take: the copy is not used, the result is the library's
-    big = rnd(100, k, dtype=torch.bfloat16, seed=3)
+    big = rnd(130, k, dtype=torch.bfloat16, seed=3)
     if not gated:
         assert torch.equal(prepared.linear(big, w), plain.linear(big, w))
     # sizes that cannot be tiled are left alone
@@ -191,7 +191,7 @@ def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
     assert prepared._tiled_copy(odd) is None
 
 
-@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 70])
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 70, 128, 129])
 @pytest.mark.parametrize("n,k", [(2560, 4096), (2560, 9728), (96, 2048), (6144, 2560), (64, 64), (4096, 12288)])
 def test_product_for_the_residual_may_come_in_planes(m, n, k):
     """linear_for_residual's planes sum to the product, and add_rmsnorm adds them like one delta."""
@@ -203,7 +203,7 @@ def test_product_for_the_residual_may_come_in_planes(m, n, k):
     ops.prepare_weight(w)
     want = x.double() @ w.double().T
     got = ops.linear_for_residual(x, w)
-    if m <= 64 and ops.choose_k_parts(n, k, m) > 1:
+    if m <= 128 and ops.choose_k_parts(n, k, m) > 1:
         assert got.dim() == 3 and got.shape[0] == ops.choose_k_parts(n, k, m) and got.dtype == torch.float32
         close(got.sum(0), want, 2e-3, 2e-3)
     else:
