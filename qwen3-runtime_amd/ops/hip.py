@@ -7,8 +7,9 @@ library cannot be built or loaded, construction fails. Tensors are torch
 tensors on the GPU; outputs are allocated with torch's caching allocator.
 
 Matrix products: float32 goes to the library's own fused-multiply-add kernel
-(true 32-bit). bfloat16 with few rows, or with float32 output, goes to the
-library's MFMA kernel; bfloat16 with many rows goes to the vendor BLAS through
+(true 32-bit). bfloat16 with up to 64 rows (128 for the gated product and for
+products cut along K) goes to the library's MFMA kernels, which stream the
+weights; bfloat16 with more rows goes to the vendor BLAS through
 ``torch.matmul``, as the reference leaves its products to cuBLAS
 (qwen3_runtime/models/qwen3.py:76-77,134-135).
 """
