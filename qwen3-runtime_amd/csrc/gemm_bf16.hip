@@ -558,9 +558,10 @@ extern "C" int qrt_gemm_bf16_variant(const void* a, const void* w, void* c, int 
 
 // gated = 0: C[M, N] = A W^T with W [N, K].
 // gated = 1: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A Wg^T) * (A Wu^T).
-// tiled = 1: W is stored tile-major, [rows / 16][K / 32][64 lanes][8]: lane q * 16 + i of tile
-// (r, s) holds W[16 r + i][32 s + 8 q .. + 7]; needs N % 16 == 0, K % 32 == 0, K % 64 == 0 above 16
-// rows, and M <= 64 (M <= 128 for the gated form and for K parts).
+// tiled = 1 or 2: W is stored tile-major, [rows / 16][K / 32][64 lanes][8]: lane q * 16 + i of tile
+// (r, s) holds W[16 r + i][32 s + 8 q .. + 7]; needs N % 16 == 0 and K % 32 == 0. 1: the few-row
+// kernel, M <= 16. 2: the kernel that shares the activations through LDS, K % 64 == 0 and M <= 64
+// (M <= 128 for the gated form and for K parts).
 // k_parts > 1 (tile-major, not gated, float32 out): K is cut into that many parts, each handled
 // by blocks of its own, and C is [k_parts, M, N]: planes to be added by the caller.
 extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K, int gated,
@@ -568,26 +569,31 @@ extern "C" int qrt_gemm_bf16(const void* a, const void* w, void* c, int out_dtyp
   QRT_CHECK(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   QRT_CHECK(gated == 0 || gated == 1, "gemm_bf16: unknown mode %d", gated);
   QRT_CHECK(k_parts >= 1 && k_parts <= 64, "gemm_bf16: bad number of K parts %d", k_parts);
-  QRT_CHECK(k_parts == 1 || (tiled && !gated && out_dtype == QRT_F32),
+  QRT_CHECK(k_parts == 1 || (tiled != 0 && !gated && out_dtype == QRT_F32),
             "gemm_bf16: K parts need tile-major weights, no gate and float32 output");
   if (M == 0) return 0;
   const bf16_t* A = (const bf16_t*)a;
   const bf16_t* W = (const bf16_t*)w;
   const bool aligned = (K % 32 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0);
-  if (tiled) {
-    QRT_CHECK(M <= 128 && N % 16 == 0 && aligned,
-              "gemm_bf16: tile-major weights need M <= 128, N %% 16 == 0, K %% 32 == 0 (M=%d N=%d K=%d)", M, N, K);
-    if (M <= 16)
-      return gated ? skinny_tiled<true>(A, W, c, out_dtype, M, N, K, stream, 1)
-                   : skinny_tiled<false>(A, W, c, out_dtype, M, N, K, stream, k_parts);
-    QRT_CHECK(K % 64 == 0 && N <= (1 << 20),
-              "gemm_bf16: 17 to 128 rows on tile-major weights need K %% 64 == 0 and N <= 2^20 (N=%d K=%d)", N, K);
+  if (tiled == 1) {  // the few-row kernel
+    QRT_CHECK(M <= 16 && N % 16 == 0 && aligned,
+              "gemm_bf16: the few-row kernel on tile-major weights needs M <= 16, N %% 16 == 0, K %% 32 == 0 "
+              "(M=%d N=%d K=%d)", M, N, K);
+    return gated ? skinny_tiled<true>(A, W, c, out_dtype, M, N, K, stream, 1)
+                 : skinny_tiled<false>(A, W, c, out_dtype, M, N, K, stream, k_parts);
+  }
+  if (tiled == 2) {  // the kernel that shares the activations through LDS
+    QRT_CHECK(M <= 128 && N % 16 == 0 && N <= (1 << 20) && K % 64 == 0 && aligned,
+              "gemm_bf16: the LDS-sharing kernel needs M <= 128, N %% 16 == 0, N <= 2^20, K %% 64 == 0 "
+              "(M=%d N=%d K=%d)", M, N, K);
+    if (M <= 16) return mid<1>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
     if (M <= 32) return mid<2>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
     if (M <= 48) return mid<3>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
     if (M <= 64) return mid<4>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
     if (M <= 96) return mid<6>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
     return mid<8>(A, W, c, out_dtype, M, N, K, gated, stream, k_parts);
   }
+  QRT_CHECK(tiled == 0, "gemm_bf16: unknown weight layout %d", tiled);
   if (M <= 16 && aligned) return gated ? skinny<true>(A, W, c, out_dtype, M, N, K, stream)
                                        : skinny<false>(A, W, c, out_dtype, M, N, K, stream);
   QRT_CHECK(gated == 0, "gemm_bf16: the gated form needs K a multiple of 32, and M <= 16 or tile-major weights "

@@ -140,12 +140,17 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> torch.Tensor:
 
 
 class HipOps:
-    # bfloat16 products with more rows than this go to the vendor BLAS (up to 16 rows any weight
-    # will do; from 17 rows on the own kernel wants the tile-major copy and K a multiple of 64)
+    # bfloat16 products with more rows than this go to the vendor BLAS
     own_max_rows = 64
     # the same for the two forms in which a block fetches fewer activations than weights: the
     # gated product, and the product cut along K whose planes the residual's norm adds
     own_max_rows_shared = 128
+    # Rows from which a product takes the kernel that shares the activations through LDS
+    # instead of the few-row kernel (both stream tile-major weights). Measured at the 4B
+    # shapes: cut along K the sharing kernel alone is 5 to 22 % faster from 4 rows on, gated
+    # from 12 rows on; a decode step is as fast either way at batch 8 and 5 % faster with it
+    # at batch 16.
+    shared_from_rows = {"whole": 17, "gated": 12, "planes": 9}
     # tiles of 16 rows per wave in the attention kernel for long portions (1, 2 or 4)
     prefill_row_tiles = 2
     # long portions: keys and values go through LDS, shared by the four waves of a block
@@ -242,27 +247,32 @@ class HipOps:
         if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
             raise OpsError(f"linear: no product of {x.dtype} activations with {w.dtype} weights")
         tiled = self._tiled_copy(w)
-        if not self._own_kernel_takes(m, k, tiled, self.own_max_rows):
+        kernel = self._own_kernel(m, k, tiled, "whole")
+        if kernel is None:
             # many rows: the vendor library; both accumulate in float32
             if out_f32:
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
             return torch.matmul(x, w.t())
         out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
         self._check(self.lib, self.lib.qrt_gemm_bf16(
-            _ptr(x), _ptr(w if tiled is None else tiled), _ptr(out), F32 if out_f32 else BF16,
-            c_int(m), c_int(n), c_int(k), c_int(0), c_int(0 if tiled is None else 1), c_int(1), _stream()))
+            _ptr(x), _ptr(tiled if kernel else w), _ptr(out), F32 if out_f32 else BF16,
+            c_int(m), c_int(n), c_int(k), c_int(0), c_int(kernel), c_int(1), _stream()))
         return out
 
-    @staticmethod
-    def _own_kernel_takes(m: int, k: int, tiled, max_rows: int) -> bool:
-        """Rows up to 16: the few-row kernel, on any weight layout. 17 to ``max_rows``: the
-        kernel that shares the activations through LDS, on the tile-major copy only (measured at
-        the 4B shapes, 32 and 64 rows: 28 to 32 % less time than the vendor library over the four
-        products of a layer; at 128 rows the gated product and the products cut along K take 71
-        us against the library's 116). Without the copy, or beyond, the vendor library."""
-        if m <= min(16, max_rows):
-            return True
-        return m <= max_rows and tiled is not None and k % 64 == 0
+    def _own_kernel(self, m: int, k: int, tiled, form: str) -> int | None:
+        """Which of the library's kernels multiplies ``m`` rows by this weight: 0 the few-row
+        kernel on the weight as stored, 1 the same on the tile-major copy, 2 the kernel that
+        shares the activations through LDS (tile-major copy, K a multiple of 64), None the
+        vendor library. ``form``: "whole", "gated", or "planes" (cut along K). Measured at the
+        4B shapes against the vendor library: 28 to 32 % less time over the four products of a
+        layer at 32 and 64 rows; at 128 rows 71 us against 116 for the gated product and the
+        two cut along K."""
+        limit = self.own_max_rows if form == "whole" else self.own_max_rows_shared
+        if tiled is not None and k % 64 == 0 and self.shared_from_rows[form] <= m <= limit:
+            return 2
+        if m <= min(16, limit):
+            return 0 if tiled is None else 1
+        return None
 
     def linear_for_residual(self, x, w):
         """``linear(x, w)`` for a result that is only ever added to the residual stream.
@@ -273,34 +283,33 @@ class HipOps:
         m, k = x.shape
         n = w.shape[0]
         tiled = self._tiled_copy(w) if x.dtype == torch.bfloat16 else None
-        if tiled is None or not self._own_kernel_takes(m, k, tiled, self.own_max_rows_shared):
-            return self.linear(x, w)
-        parts = self.choose_k_parts(n, k, m)
+        kernel = self._own_kernel(m, k, tiled, "planes") if tiled is not None else None
+        parts = self.choose_k_parts(n, k, m, kernel == 2) if kernel else 1
         if parts == 1:
             return self.linear(x, w)
         _need(x, "x", torch.bfloat16)
         out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
         self._check(self.lib, self.lib.qrt_gemm_bf16(
-            _ptr(x), _ptr(tiled), _ptr(out), F32, c_int(m), c_int(n), c_int(k), c_int(0), c_int(1),
+            _ptr(x), _ptr(tiled), _ptr(out), F32, c_int(m), c_int(n), c_int(k), c_int(0), c_int(kernel),
             c_int(parts), _stream()))
         return out
 
     @staticmethod
-    def choose_k_parts(n: int, k: int, m: int = 1) -> int:
-        """Up to 16 rows: cut K when there are fewer row tiles than about two per compute unit
-        and K is long. 17 to 128 rows: a block takes up to six row tiles, so that they share the
-        activations, and K is cut until there are about as many blocks as compute units, each
-        part keeping 12 k-steps or more."""
+    def choose_k_parts(n: int, k: int, m: int = 1, shared: bool | None = None) -> int:
+        """The few-row kernel: cut K when there are fewer row tiles than about two per compute
+        unit and K is long. The kernel that shares activations (``shared``; by default from 17
+        rows on): a block takes up to six row tiles, and K is cut until there are about as
+        many blocks as compute units, each part keeping 12 k-steps or more."""
         tiles = n // 16
-        if m <= 16:
+        if shared is None:
+            shared = m > 16
+        if not shared:
             if tiles >= 384 or k < 2048:
                 return 1
             return 2 if k < 8192 else 4
         blocks = (tiles + 5) // 6
         return max(1, min(8, 256 // blocks, (k // 32) // 12))
 
-    # rows up to which the gated activation is fused into the product before it
-    fused_gate_max_rows = 128
 
     def gated_linear(self, x, w_gate_up):
         """``swiglu(linear(x, w_gate_up))`` with ``w_gate_up`` [2I, K], gate rows first. With few
@@ -310,16 +319,16 @@ class HipOps:
         two_i, kw = w_gate_up.shape
         if k != kw or two_i % 2:
             raise OpsError(f"gated_linear: x is {tuple(x.shape)}, weight is {tuple(w_gate_up.shape)}")
-        if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and m <= self.fused_gate_max_rows
-                and k % 32 == 0):
+        if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and k % 32 == 0:
             _need(x, "x")
             _need(w_gate_up, "weight")
             tiled = self._tiled_copy(w_gate_up) if (two_i // 2) % 16 == 0 else None
-            if self._own_kernel_takes(m, k, tiled, self.fused_gate_max_rows):
+            kernel = self._own_kernel(m, k, tiled, "gated")
+            if kernel is not None:
                 out = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
                 self._check(self.lib, self.lib.qrt_gemm_bf16(
-                    _ptr(x), _ptr(w_gate_up if tiled is None else tiled), _ptr(out), BF16, c_int(m),
-                    c_int(two_i // 2), c_int(k), c_int(1), c_int(0 if tiled is None else 1), c_int(1), _stream()))
+                    _ptr(x), _ptr(tiled if kernel else w_gate_up), _ptr(out), BF16, c_int(m),
+                    c_int(two_i // 2), c_int(k), c_int(1), c_int(kernel), c_int(1), _stream()))
                 return out
         return self.swiglu(self.linear(x, w_gate_up))
 

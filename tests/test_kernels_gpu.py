@@ -125,7 +125,6 @@ def test_gemm_bf16(ops, m, n, k, out_f32):
                                    (5, 64, 48), (16, 1000, 128)])
 def test_gated_linear(ops, m, i, k, monkeypatch):
     """The fused form (few rows) and the two-kernel form agree with the plain one."""
-    monkeypatch.setattr(ops, "fused_gate_max_rows", 64)
     for dtype in (torch.bfloat16, torch.float32):
         x, w = rnd(m, k, dtype=dtype, seed=3), rnd(2 * i, k, dtype=dtype, seed=4, scale=0.05)
         gu = x.double() @ w.double().T
@@ -158,7 +157,7 @@ def test_gemm_bf16_few_rows_at_model_sizes(m, n, k, prepared):
     close(ops.linear(x, w), want, 3e-2, 3e-2)
 
 
-@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 31, 33, 48, 64, 65, 96, 128])
+@pytest.mark.parametrize("m", [1, 3, 8, 11, 12, 16, 17, 31, 33, 48, 64, 65, 96, 128])
 @pytest.mark.parametrize("n,k,gated", [(6144, 2560, False), (2560, 4096, False), (608, 9728, False), (64, 64, False),
                                        (9728, 2560, True), (48, 96, True), (151936, 256, False), (80, 128, True),
                                        (4112, 640, True), (16, 64, False)])
@@ -191,7 +190,7 @@ def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
     assert prepared._tiled_copy(odd) is None
 
 
-@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 70, 128, 129])
+@pytest.mark.parametrize("m", [1, 3, 8, 9, 16, 17, 40, 64, 70, 128, 129])
 @pytest.mark.parametrize("n,k", [(2560, 4096), (2560, 9728), (96, 2048), (6144, 2560), (64, 64), (4096, 12288)])
 def test_product_for_the_residual_may_come_in_planes(m, n, k):
     """linear_for_residual's planes sum to the product, and add_rmsnorm adds them like one delta."""
@@ -203,8 +202,11 @@ def test_product_for_the_residual_may_come_in_planes(m, n, k):
     ops.prepare_weight(w)
     want = x.double() @ w.double().T
     got = ops.linear_for_residual(x, w)
-    if m <= 128 and ops.choose_k_parts(n, k, m) > 1:
-        assert got.dim() == 3 and got.shape[0] == ops.choose_k_parts(n, k, m) and got.dtype == torch.float32
+    kernel = ops._own_kernel(m, k, ops._tiled_copy(w), "planes")
+    parts = ops.choose_k_parts(n, k, m, kernel == 2) if kernel else 1
+    assert (kernel == 2) == (9 <= m <= 128 and k % 64 == 0)
+    if parts > 1:
+        assert got.dim() == 3 and got.shape[0] == parts and got.dtype == torch.float32
         close(got.sum(0), want, 2e-3, 2e-3)
     else:
         assert got.dim() == 2
