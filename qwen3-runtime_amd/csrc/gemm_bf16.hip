@@ -473,7 +473,9 @@ static int launch_mid(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, 
   constexpr int WT = GATED ? 2 * NT : NT;
   const int per_block = NWV * NT, tiles = N / 16;
   // as many blocks as compute units where the tiles allow it, each with its even share
-  int blocks = tiles <= 256 / k_parts ? tiles : max(256 / k_parts, (tiles + per_block - 1) / per_block);
+  constexpr int COMPUTE_UNITS = 256;  // of an MI355X
+  int blocks = tiles <= COMPUTE_UNITS / k_parts ? tiles
+                                                : max(COMPUTE_UNITS / k_parts, (tiles + per_block - 1) / per_block);
   blocks = max(blocks, (tiles + per_block - 1) / per_block);
   dim3 grid(blocks, k_parts), block(64 * KW * NWV);
   const size_t stage = (size_t)KW * 2 * KC * (MB * 4 * (256 + 16) + 64);
