@@ -111,6 +111,37 @@ def test_many_requests_decode_together_at_model_sizes(sized_folders, live):
     check_rounding_noise(got, {k: want_all[k] for k in got})
 
 
+def test_long_context_decode_beside_a_prompt_portion(sized_folders, monkeypatch):
+    """Decoded tokens of a request that holds 1,100 keys in the same steps as portions of another
+    request's prompt: attention then runs as two launches (the decode kernel with its keys cut
+    over blocks, the prompt kernels for the portion). Against the plain implementation."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    cfg, folder = sized_folders["qwen3_4b"]
+    reqs = traces.make_requests(cfg.vocab_size, [1106, 150], seed=12)
+    long_ids, other = reqs["r0"], reqs["r1"]
+    steps = [{"entries": [{"id": "r0", "tokens": long_ids[:1100], "want": [1099]}], "end": []}]
+    cuts = [0, 40, 70, 100, 120, 137, 150]
+    for i in range(6):
+        steps.append({"entries": [{"id": "r0", "tokens": long_ids[1100 + i: 1101 + i], "want": [0]},
+                                  {"id": "r1", "tokens": other[cuts[i]: cuts[i + 1]],
+                                   "want": list(range(cuts[i + 1] - cuts[i]))}],
+                      "end": ["r0", "r1"] if i == 5 else []})
+    steps = traces._number(steps)
+    launches = []
+    inner = HipOps._launch_attention
+    monkeypatch.setattr(HipOps, "_launch_attention",
+                        lambda self, *a: (launches.append(a[-2:]), inner(self, *a))[1])
+    engine_cfg = EngineConfig(page_size=16, num_pages=traces.peak_tokens(steps) // 16, max_num_seqs=4, dtype="bfloat16",
+                              device="cuda:0", hip_graph=False)
+    got = traces.replay(load(folder, engine_cfg), steps)
+    assert ([0], True) in launches and ([1], False) in launches, "the mixed steps ran as two launches"
+    want = traces.plain_logits(folder, reqs)
+    check_rounding_noise(got, {k: want[k] for k in got})
+
+
 def test_model_sized_decode_graph_equals_eager(sized_folders):
     """Greedy tokens of three requests at the 4B layer sizes: replayed HIP graphs give the tokens
     of eager steps."""
