@@ -66,3 +66,34 @@ def test_step_refuses_bad_entries(model_folders, tiny_configs):
         loaded.runner.step([StepEntry("a", list(range(3 * page)))])
     assert loaded.cache.length("a") == 0
     loaded.cache.check()
+
+
+def test_which_kernel_multiplies_how_many_rows():
+    """The host's choice between the few-row kernel, the kernel that shares activations through
+    LDS and the vendor library, by form of the product and number of rows; and the attention work
+    list: every row of every sequence once, longest tiles first, the subset's own sequence ids."""
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    ops = HipOps.__new__(HipOps)          # the choices need no library and no GPU
+    copy = object()                       # stands for a tile-major copy
+    assert [ops._own_kernel(m, 2560, copy, "whole") for m in (1, 16, 17, 64, 65)] == [1, 1, 2, 2, None]
+    assert [ops._own_kernel(m, 2560, copy, "gated") for m in (1, 11, 12, 64, 128, 129)] == [1, 1, 2, 2, 2, None]
+    assert [ops._own_kernel(m, 4096, copy, "planes") for m in (1, 8, 9, 128, 129)] == [1, 1, 2, 2, None]
+    assert [ops._own_kernel(m, 2560, None, "whole") for m in (1, 16, 17)] == [0, 0, None]   # no copy
+    assert [ops._own_kernel(m, 96, copy, "planes") for m in (8, 16, 17)] == [1, 1, None]    # K no multiple of 64
+    # the few-row kernel cuts K when there are few row tiles; the sharing kernel until the chip is full
+    assert HipOps.choose_k_parts(2560, 4096, 8) == 2 and HipOps.choose_k_parts(2560, 9728, 8) == 4
+    assert HipOps.choose_k_parts(6144, 2560, 8) == 1 and HipOps.choose_k_parts(2560, 64, 8) == 1
+    assert HipOps.choose_k_parts(2560, 4096, 64) == 8 and HipOps.choose_k_parts(2560, 4096, 12, True) == 8
+    assert HipOps.choose_k_parts(2560, 384, 64) == 1 and HipOps.choose_k_parts(65536, 4096, 64) == 1
+
+    q_lens, kv_lens, g = [70, 1, 33], [200, 900, 33], 4
+    tiles, n = HipOps.plan_tiles(q_lens, kv_lens, g, 64, nkv=2)
+    seqs, row0 = tiles[:n].tolist(), tiles[n: 2 * n].tolist()
+    covered = {}
+    for s, r in zip(seqs, row0):
+        covered.setdefault(s, []).append(r)
+    assert {s: sorted(r) for s, r in covered.items()} == {0: [0, 64, 128, 192, 256], 1: [0], 2: [0, 64, 128]}
+    assert seqs[0] == 1                  # the tile that sees 900 keys goes first
+    sub, n_sub = HipOps.plan_tiles([70, 33], [200, 33], g, 64, nkv=2, seq_ids=[0, 2])
+    assert sorted(set(sub[:n_sub].tolist())) == [0, 2]
