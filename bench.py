@@ -93,7 +93,7 @@ def main() -> int:
         prompts = torch.randint(0, cfg.vocab_size, (batch, args.prompt_len), generator=gen).tolist()
         reqs = [engine.request(engine.add_request(p, max_tokens=k + w + lead(batch) + 8, sampling=SamplingParams()))
                 for p in prompts]
-        while any(len(r.token_ids) == r.num_prompt_tokens for r in reqs):
+        while any(len(r.token_ids) == r.prompt_len for r in reqs):
             engine.step()  # prompt portions until every request has its first token
         for _ in range(w):
             engine.step()

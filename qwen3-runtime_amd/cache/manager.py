@@ -72,6 +72,10 @@ class CacheManager:
         self._state_of_cache: dict[int, torch.Tensor] = {}
         self._length: dict[Hashable, int] = {}
         self._reserved: dict[Hashable, int] = {}
+        # Counts the events after which a block table kept elsewhere no longer describes its
+        # request: pages dropped (end, restart) and a request id admitted (possibly again).
+        # Whoever keeps a packed copy of tables compares this number before trusting the copy.
+        self.epoch = 0
         by_key: dict[tuple, _Group] = {}
         for cid, spec in enumerate(self.specs):
             if spec.kind == "paged_kv":
@@ -127,6 +131,7 @@ class CacheManager:
         if rid in self._length:
             raise AssertionError(f"request {rid!r} is admitted twice")
         slot = self.slots.take(rid)
+        self.epoch += 1
         self._length[rid] = 0
         self._reserved[rid] = 0
         for g in self.groups:
@@ -183,6 +188,7 @@ class CacheManager:
             g.first_live[rid] = i
 
     def _drop_pages(self, rid: Hashable) -> None:
+        self.epoch += 1
         for g in self.groups:
             for page in g.tables[rid]:
                 if page >= 0:

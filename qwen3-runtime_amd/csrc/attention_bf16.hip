@@ -796,7 +796,18 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   if (a.num_tiles == 0) return 0;
   const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
   dim3 grid(a.num_tiles, a.nkv, a.num_splits), block(64 * DW);
-  const size_t smem = (size_t)(2 * DW * 16 + DW * 16 * D) * sizeof(float);
+  constexpr size_t smem = (size_t)(2 * DW * 16 + DW * 16 * D) * sizeof(float);
+  if (smem > 64 * 1024) {  // head size 256: a little more LDS than a block gets without asking
+    static bool allowed = false;  // once: not again inside every stream capture
+    if (!allowed) {
+      if (hipFuncSetAttribute((const void*)attention_bf16_decode_kernel<true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess ||
+          hipFuncSetAttribute((const void*)attention_bf16_decode_kernel<false>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return qrt_fail("attention (decode): cannot get %zu bytes of LDS", smem);
+      allowed = true;
+    }
+  }
   if (p2) attention_bf16_decode_kernel<true><<<grid, block, smem, stream>>>(a);
   else attention_bf16_decode_kernel<false><<<grid, block, smem, stream>>>(a);
   QRT_LAUNCH_CHECK("attention_bf16_decode");
@@ -809,8 +820,6 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   }
   return 0;
 }
-
-extern "C" int qrt_attention_bf16_head_dim() { return D; }
 
 extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, hipStream_t stream) {
   AttnTileArgs a = *args;
@@ -837,8 +846,6 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   else if (a.row_tiles == 1) attention_bf16_kernel<1, false><<<grid, block, 0, stream>>>(a);
   else if (a.row_tiles == 2 && p2) attention_bf16_kernel<2, true><<<grid, block, 0, stream>>>(a);
   else if (a.row_tiles == 2) attention_bf16_kernel<2, false><<<grid, block, 0, stream>>>(a);
-  else if (a.row_tiles == 4 && D <= 128 && p2) attention_bf16_kernel<4, true><<<grid, block, 0, stream>>>(a);
-  else if (a.row_tiles == 4 && D <= 128) attention_bf16_kernel<4, false><<<grid, block, 0, stream>>>(a);
   else return qrt_fail("attention: %d row tiles per wave at head size %d is not built", a.row_tiles, D);
   QRT_LAUNCH_CHECK("attention_bf16");
   if (a.num_splits > 1) {

@@ -535,29 +535,6 @@ static int launch(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int 
   return 0;
 }
 
-// Tuning aid: run one named configuration of the few-row kernel (M <= 16), so that
-// configurations can be timed against each other on the shapes of a model.
-extern "C" int qrt_gemm_bf16_variant(const void* a, const void* w, void* c, int out_dtype, int M, int N, int K,
-                                     int gated, int variant, hipStream_t stream) {
-  QRT_CHECK(M >= 1 && M <= 16 && K % 32 == 0, "gemm_bf16_variant: M <= 16 and K a multiple of 32 only");
-  const bf16_t* A = (const bf16_t*)a;
-  const bf16_t* W = (const bf16_t*)w;
-#define V(ID, NW, NT, U)                                                                            \
-  if (variant == ID)                                                                                \
-    return gated ? launch_skinny<1, NW, NT, U, true>(A, W, c, out_dtype, M, N, K, stream)           \
-                 : launch_skinny<1, NW, NT, U, false>(A, W, c, out_dtype, M, N, K, stream);
-  V(0, 8, 1, 8) V(1, 8, 2, 8) V(2, 16, 1, 8) V(4, 4, 1, 8) V(10, 4, 1, 16)
-#undef V
-  // 100 + id: the same on tile-major weights
-#define V(ID, NW, NT, U)                                                                            \
-  if (variant == 100 + ID)                                                                          \
-    return gated ? launch_skinny<1, NW, NT, U, true, true>(A, W, c, out_dtype, M, N, K, stream)     \
-                 : launch_skinny<1, NW, NT, U, false, true>(A, W, c, out_dtype, M, N, K, stream);
-  V(0, 8, 1, 8) V(1, 8, 2, 8) V(2, 16, 1, 8) V(4, 4, 1, 8) V(10, 4, 1, 16)
-#undef V
-  return qrt_fail("gemm_bf16_variant: no variant %d", variant);
-}
-
 // gated = 0: C[M, N] = A W^T with W [N, K].
 // gated = 1: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A Wg^T) * (A Wu^T).
 // tiled = 1 or 2: W is stored tile-major, [rows / 16][K / 32][64 lanes][8]: lane q * 16 + i of tile

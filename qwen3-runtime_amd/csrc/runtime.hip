@@ -14,5 +14,3 @@ int qrt_fail(const char* fmt, ...) {
   va_end(ap);
   return -1;
 }
-
-extern "C" int qrt_abi_version() { return 1; }

@@ -139,7 +139,7 @@ __device__ __forceinline__ void first_pass(const RowOptions& o, const float* __r
       ssum = ssum * expf(m - v) + 1.0f;  // m = -inf at first: exp(-inf) = 0
       m = v;
       bi = i;
-    } else if (v == v) {
+    } else if (v > -INFINITY) {  // neither NaN nor an excluded id (-inf beside m = -inf would give NaN)
       ssum += expf(v - m);
     }
     return v;
@@ -383,7 +383,7 @@ extern "C" int qrt_sample(const SampleArgs* args, hipStream_t stream) {
 // counts[slot[i], token[i]] += 1   (ids a request has seen: prompt and output)
 __global__ void count_tokens_kernel(int* counts, const int* slot, const int* token, int n, int vocab) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) atomicAdd(&counts[(size_t)slot[i] * vocab + token[i]], 1);
+  if (i < n && token[i] >= 0 && token[i] < vocab) atomicAdd(&counts[(size_t)slot[i] * vocab + token[i]], 1);
 }
 
 extern "C" int qrt_count_tokens(int* counts, const int* slot, const int* token, int n, int vocab, hipStream_t stream) {
@@ -396,7 +396,7 @@ extern "C" int qrt_count_tokens(int* counts, const int* slot, const int* token, 
 // logits[row[i], token[i]] += value[i]   (logit bias; reference: qwen3_runtime/sampling.py:35-41)
 __global__ void add_bias_kernel(float* logits, const int* row, const int* token, const float* value, int n, int vocab) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) atomicAdd(&logits[(size_t)row[i] * vocab + token[i]], value[i]);
+  if (i < n && token[i] >= 0 && token[i] < vocab) atomicAdd(&logits[(size_t)row[i] * vocab + token[i]], value[i]);
 }
 
 extern "C" int qrt_add_bias(float* logits, const int* row, const int* token, const float* value, int n, int vocab,

@@ -1,22 +1,23 @@
-"""The engine loop: schedule, run one step, sample, finish.
+"""The engine loop: decide a step, run it, sample, settle.
 
-``add_request`` queues a request; ``step()`` asks the scheduler for a batch,
-runs it through the step function, samples the rows that reached the end of
-their tokens and returns ``[(request id, new token or None, finished)]``
-(reference: qwen3_runtime/engine/engine.py:53-92,216-260).
+``add_request`` queues a request and returns its id. ``step()`` asks the
+scheduler who takes part, hands their next tokens to the step function, samples
+for every request whose tokens are now all in the cache, and reports
+``[(request id, new token or None, ended)]`` (reference, for the same contract:
+qwen3_runtime/engine/engine.py:53-92,216-260). ``generate`` and
+``generate_batch`` drive ``step()`` until their requests have ended.
 """
 
 from __future__ import annotations
 
+import math
 from typing import Iterator, Sequence
-
-import torch
 
 from ..config.engine import EngineConfig
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
-from .request import Request, RequestStatus
+from .request import Request
 from .scheduler import Scheduler
 
 
@@ -26,138 +27,142 @@ class Engine:
         self.loaded = loaded
         self.cache = loaded.cache
         self.runner = loaded.runner
-        self.scheduler = Scheduler(config, self.cache, self.runner.max_model_len)
+        self.scheduler = Scheduler(config, self.cache, self.runner.max_model_len,
+                                   portion_multiple=loaded.model.portion_multiple)
         self.sampler = Sampler(self.runner.ops, self.cache.slots, self.runner.vocab_size, self.runner.device)
-        self._requests: dict[int, Request] = {}
+        self._live: dict[int, Request] = {}
         self.last_step_stats: dict | None = None
-        self._fatal_error: str | None = None
+        self._broken: str | None = None
 
-    # ---- requests --------------------------------------------------------------
-    def add_request(
-        self,
-        token_ids: Sequence[int],
-        max_tokens: int = 16,
-        *,
-        ignore_eos: bool = True,
-        sampling: SamplingParams | None = None,
-        stop_token_ids: Sequence[int] = (),
-        forced_tokens: Sequence[int] | None = None,
-    ) -> int:
-        self._check_health()
-        req = Request(token_ids, max_tokens, ignore_eos, sampling=sampling,
-                      stop_token_ids=stop_token_ids, forced_tokens=forced_tokens)
-        bad = [t for t in req.token_ids if not 0 <= t < self.runner.vocab_size]
-        if bad:
-            raise ValueError(f"token id {bad[0]} is outside the vocabulary of {self.runner.vocab_size}")
+    # ---- requests ----------------------------------------------------------------
+    def add_request(self, token_ids: Sequence[int], max_tokens: int = 16, *, ignore_eos: bool = True,
+                    sampling: SamplingParams | None = None, stop_token_ids: Sequence[int] = (),
+                    forced_tokens: Sequence[int] | None = None) -> int:
+        self._refuse_if_broken()
+        req = Request(token_ids, max_tokens, ignore_eos, sampling=sampling, stop_token_ids=stop_token_ids,
+                      forced_tokens=forced_tokens)
+        self._check_ids(req)
         self.scheduler.add(req)
-        self._requests[req.request_id] = req
+        self._live[req.request_id] = req
         return req.request_id
 
+    def _check_ids(self, req: Request) -> None:
+        """Every id that will index device memory (the embedding table, a row of logits, the
+        penalty counts) is checked here, on the host: a kernel cannot report a bad index, it
+        can only write where it must not."""
+        vocab = self.runner.vocab_size
+        bias = req.sampling.logit_bias or {}
+        for what, ids in (("prompt token", req.token_ids), ("forced token", req.forced or ()),
+                          ("logit_bias key", list(bias))):
+            for t in ids:
+                if isinstance(t, bool) or int(t) != t or not 0 <= int(t) < vocab:
+                    raise ValueError(f"{what} {t!r} is outside the vocabulary of {vocab} ids")
+        for t, v in bias.items():
+            v = float(v)
+            if math.isnan(v) or v == math.inf:
+                raise ValueError(f"logit_bias[{t}] = {v}: a bias is a finite number, or -inf to exclude the id")
+
     def request(self, request_id: int) -> Request:
-        return self._requests[request_id]
+        return self._live[request_id]
 
     def finish_request(self, request_id: int) -> None:
-        """Cancel: give back what the request holds."""
-        req = self._requests.pop(request_id, None)
-        if req is not None and req.status != RequestStatus.FINISHED:
-            req.finish_reason = req.finish_reason or "abort"
-            self.scheduler.finish(req)
+        """Cancel: the request ends now and gives back what it holds."""
+        req = self._live.pop(request_id, None)
+        if req is not None:
+            self.scheduler.retire(req, "abort")
 
     def is_finished(self) -> bool:
         return self.scheduler.is_finished()
 
-    # ---- one step -----------------------------------------------------------------
-    def _check_health(self) -> None:
-        """After a failure on the device side of a step the cache's books and the device's state
-        no longer agree: the engine refuses further work
+    # ---- one step -------------------------------------------------------------------
+    def _refuse_if_broken(self) -> None:
+        """A step that failed on the device side leaves the cache's books and the device's
+        contents in disagreement; nothing more is run on them
         (reference: qwen3_runtime/engine/engine.py:210-225)."""
-        if self._fatal_error is not None:
-            raise RuntimeError("engine terminated after a failed step: " + self._fatal_error)
+        if self._broken is not None:
+            raise RuntimeError("engine terminated after a failed step: " + self._broken)
 
     def step(self) -> list[tuple[int, int | None, bool]]:
-        self._check_health()
-        preempt_before = self.scheduler.num_preemptions
-        reqs = self.scheduler.schedule()
-        if not reqs:
+        self._refuse_if_broken()
+        evictions = self.scheduler.num_preemptions
+        batch = self.scheduler.schedule()
+        if not batch:
             self.last_step_stats = None
             if not self.scheduler.is_finished():
                 raise RuntimeError("scheduler produced an empty step while requests remain")
             return []
-        entries, sampling_reqs = [], []
-        prefill_tokens = decode_tokens = 0
-        for req in reqs:
-            start = self.cache.length(req.request_id)
-            n = req.num_scheduled_tokens
-            if start == 0 and req.num_preemptions == 0:
-                self.sampler.admit(self.cache.slots.slot(req.request_id), req.sampling, req.seed,
-                                   req.token_ids[: req.num_prompt_tokens])
-            reaches_end = start + n >= len(req.token_ids)
-            entries.append(StepEntry(req.request_id, req.token_ids[start: start + n],
-                                     [n - 1] if reaches_end else []))
-            if reaches_end:
-                sampling_reqs.append(req)
-            if start >= req.num_prompt_tokens:
-                decode_tokens += n
-            else:
-                prefill_tokens += n
         try:
-            return self._run(reqs, entries, sampling_reqs, prefill_tokens, decode_tokens, preempt_before)
+            return self._run_step(batch, evictions)
         except BaseException as exc:
-            self._fatal_error = f"{type(exc).__name__}: {exc}"
+            self._broken = f"{type(exc).__name__}: {exc}"
             raise
 
-    def _run(self, reqs, entries, sampling_reqs, prefill_tokens, decode_tokens, preempt_before):
+    def _run_step(self, batch: list[Request], evictions_before: int):
+        entries, to_sample = [], []
+        n_prompt = n_decode = 0
+        for req in batch:
+            at = self.cache.length(req.request_id)
+            if at == 0 and req.restarts == 0:  # its first step: options and seed go into its slot
+                self.sampler.admit(self.cache.slots.slot(req.request_id), req.sampling, req.seed,
+                                   req.token_ids[: req.prompt_len])
+            upto = at + req.grant
+            caught_up = upto >= len(req.token_ids)
+            entries.append(StepEntry(req.request_id, req.token_ids[at:upto], [req.grant - 1] if caught_up else []))
+            if caught_up:
+                to_sample.append(req)
+            if at >= req.prompt_len:
+                n_decode += req.grant
+            else:
+                n_prompt += req.grant
         logits = self.runner.step(entries)
-        tokens: list[int | None] = [None] * len(reqs)
-        if sampling_reqs:
-            # the rows' state slots went up with the step's other arrays: no copy, no wait here
+        new_token: dict[int, int] = {}
+        if to_sample:
+            # the rows' state slots went to the device with the step's other arrays
             slot_rows = self.runner.last_row_slots
-            if slot_rows is None or slot_rows.numel() != len(sampling_reqs):
+            if logits is None or slot_rows is None or slot_rows.numel() != len(to_sample):
                 raise RuntimeError("the step's logits do not match the requests to sample for")
-            sampled, logprobs = self.sampler.sample(logits, slot_rows, sampling_reqs)
-            by_id = {r.request_id: (t, lp) for r, t, lp in zip(sampling_reqs, sampled, logprobs)}
-            for i, req in enumerate(reqs):
-                if req.request_id in by_id:
-                    tokens[i], lp = by_id[req.request_id]
-                    req.logprobs.append(lp)
-        finished = {r.request_id for r in self.scheduler.postprocess(reqs, tokens)}
+            ids, logprobs = self.sampler.sample(logits, slot_rows, to_sample)
+            for req, tok, lp in zip(to_sample, ids, logprobs):
+                new_token[req.request_id] = tok
+                req.logprobs.append(lp)
+        sampled = [new_token.get(req.request_id) for req in batch]
+        ended = {req.request_id for req in self.scheduler.settle(batch, sampled)}
+        for rid in ended:
+            self._live.pop(rid, None)
         self.last_step_stats = {
-            "req_ids": [r.request_id for r in reqs],
-            "prefill_tokens": prefill_tokens,
-            "decode_tokens": decode_tokens,
-            "preempts": self.scheduler.num_preemptions - preempt_before,
+            "req_ids": [req.request_id for req in batch],
+            "prefill_tokens": n_prompt,
+            "decode_tokens": n_decode,
+            "preempts": self.scheduler.num_preemptions - evictions_before,
         }
-        for rid in finished:
-            self._requests.pop(rid, None)
-        return [(r.request_id, t, r.request_id in finished) for r, t in zip(reqs, tokens)]
+        return [(req.request_id, tok, req.request_id in ended) for req, tok in zip(batch, sampled)]
 
-    # ---- whole requests --------------------------------------------------------------
+    # ---- whole requests ------------------------------------------------------------------
+    def _drive(self, reqs: Sequence[Request]) -> Iterator[list[tuple[int, int | None, bool]]]:
+        while not all(r.done for r in reqs):
+            results = self.step()
+            if not results:
+                raise RuntimeError("no progress while requests remain")
+            yield results
+
     def stream_request(self, request_id: int) -> Iterator[int]:
-        """Yield the request's new tokens until it finishes (other requests advance too)."""
-        req = self._requests[request_id]
-        while req.status != RequestStatus.FINISHED:
-            progressed = False
-            for rid, tok, _done in self.step():
-                progressed = True
+        """The request's new tokens as they come (other queued requests advance as well)."""
+        for results in self._drive([self._live[request_id]]):
+            for rid, tok, _ended in results:
                 if rid == request_id and tok is not None:
                     yield tok
-            if not progressed:
-                raise RuntimeError(f"request {request_id} made no progress")
 
-    def generate(self, token_ids: Sequence[int], max_tokens: int = 16, **kwargs) -> list[int]:
-        return list(self.stream_request(self.add_request(token_ids, max_tokens=max_tokens, **kwargs)))
+    def generate(self, token_ids: Sequence[int], max_tokens: int = 16, **options) -> list[int]:
+        return list(self.stream_request(self.add_request(token_ids, max_tokens=max_tokens, **options)))
 
     def generate_batch(self, prompts: Sequence[Sequence[int]], max_tokens: int = 16, sampling=None,
-                       **kwargs) -> list[list[int]]:
+                       **options) -> list[list[int]]:
         """All prompts are queued at once and batched continuously; outputs in the order given."""
-        samplings = sampling if isinstance(sampling, (list, tuple)) else [sampling] * len(prompts)
-        reqs = []
-        for p, s in zip(prompts, samplings):
-            rid = self.add_request(p, max_tokens=max_tokens, sampling=s, **kwargs)
-            reqs.append(self._requests[rid])
-        while any(r.status != RequestStatus.FINISHED for r in reqs):
-            if not self.step():
-                raise RuntimeError("no progress while requests remain")
+        per_prompt = sampling if isinstance(sampling, (list, tuple)) else [sampling] * len(prompts)
+        reqs = [self._live[self.add_request(p, max_tokens=max_tokens, sampling=s, **options)]
+                for p, s in zip(prompts, per_prompt)]
+        for _ in self._drive(reqs):
+            pass
         return [r.output_tokens for r in reqs]
 
     def config_report(self) -> dict:

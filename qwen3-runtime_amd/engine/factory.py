@@ -41,11 +41,20 @@ def build_model(raw_config: dict) -> tuple[object, DecoderModel]:
 
 
 def pages_for_memory(model: DecoderModel, engine: EngineConfig, dtype: torch.dtype, device) -> int:
+    """Pages per group when none were asked for: what ``memory_fraction`` of the free device
+    memory holds, but never more than the engine can use. ``max_num_seqs`` requests can be
+    resident, each at most ``max_model_len`` tokens long, so more pages than that (plus one
+    spare page per request) would only be memory taken from everything else: a small model
+    would otherwise claim most of the device, and the host lists with one entry per page
+    would have millions of entries. At least 32 pages, as the reference
+    (qwen3_runtime/engine/factory.py:94-107)."""
     per_page = CacheManager.bytes_per_page(model.plan.caches, engine.page_size, torch.finfo(dtype).bits // 8)
     if per_page == 0:
         return 32
+    max_len = min(engine.max_model_len or model.plan.max_positions, model.plan.max_positions)
+    useful = engine.max_num_seqs * (-(-max_len // engine.page_size) + 1)
     free, _total = torch.cuda.mem_get_info(device)
-    return max(32, int(free * engine.memory_fraction) // per_page)
+    return max(32, min(useful, int(free * engine.memory_fraction) // per_page))
 
 
 def copies_fit(model: DecoderModel, engine: EngineConfig, dtype: torch.dtype, device) -> bool:

@@ -49,6 +49,7 @@ class DecodeGraph:
         # what the host buffer holds: the requests of the last fill and their lengths before it
         self._last_rids: list | None = None
         self._last_starts: list[int] | None = None
+        self._last_epoch = -1  # the cache's epoch at the last fill: a later one voids the buffer
         self._host_views = None
         self._row_index = None
 
@@ -56,13 +57,16 @@ class DecodeGraph:
         runner = self.runner
         rids = [e.request_id for e in entries]
         starts = [runner.cache.length(r) for r in rids]
-        if self.graph is not None and rids == self._last_rids:
+        # The kept buffer is only good while no request has dropped pages or been admitted since:
+        # the same id at the same length may by then own other pages (restart after preemption,
+        # release and a new request under the old id).
+        if self.graph is not None and rids == self._last_rids and runner.cache.epoch == self._last_epoch:
             if starts != self._last_starts and all(a == b + 1 for a, b in zip(starts, self._last_starts)):
                 self._advance(rids, starts)
             if starts == self._last_starts:  # the buffer holds this step, but for the ids
                 self._send(entries)
                 return None
-        self._last_rids, self._last_starts = rids, starts
+        self._last_rids, self._last_starts, self._last_epoch = rids, starts, runner.cache.epoch
         packed = pack_step(entries, runner.cache, runner.vocab_size, table_width=self.width)
         if self.layout is None:
             off, layout = 0, []
@@ -136,6 +140,8 @@ class DecodeGraph:
         if self.graph is None or self._last_rids is None:
             return
         cache, rids = self.runner.cache, self._last_rids
+        if cache.epoch != self._last_epoch or not all(cache.has(r) for r in rids):
+            return
         starts = [cache.length(r) for r in rids]
         if any(a != b + 1 for a, b in zip(starts, self._last_starts)):
             return

@@ -35,7 +35,8 @@ class ModelRunner:
         self.device = torch.device(device)
         self.max_model_len = int(max_model_len or model.plan.max_positions)
         self.vocab_size = model.plan.vocab_size
-        self.hip_graph = bool(hip_graph) and self.device.type == "cuda"
+        # graphs only where every part of the model can be captured (a part says so itself)
+        self.hip_graph = bool(hip_graph) and self.device.type == "cuda" and model.graph_capturable
         self._graphs: dict[tuple, "_DecodeGraph"] = {}
         self._graph_pool = None
         # device copy of the last step's "row_slots" (state slot of each row of the logits)

@@ -1,21 +1,25 @@
-"""Continuous batching with prompts cut into portions under a token budget.
+"""Who takes part in the next step, and with how many tokens.
 
-One ``schedule()`` call decides a step: running requests first, in admission
-order (a decoding request takes one token, an unfinished prompt a portion),
-then waiting requests while the token budget and ``max_num_seqs`` allow. A
-portion is ``min(uncomputed, budget)``, shrunk to what the request's held pages
-plus the free pages can store. Pages are reserved only for the step's tokens
-(reference: qwen3_runtime/engine/scheduler.py:47-64,227-295).
+A step has two limits: ``max_num_batched_tokens`` tokens and ``max_num_seqs``
+requests. Candidates are walked in one fixed order, residents (requests that
+hold pages, oldest first) and then the queue (arrival order), and each is
+offered ``min(what it still has to compute, what is left of the token limit)``,
+cut down to the tokens its own pages plus the free pages can hold. A decoding
+request therefore takes one token and a prompt is cut into portions; pages are
+taken for the step's tokens only. These are the reference's rules
+(qwen3_runtime/engine/scheduler.py:47-64,227-295); the walk over one candidate
+list is this file's own.
 
-When pages run out: a running request that cannot get a page sits the step
-out. If no request at all can be scheduled, the youngest running request is
-preempted: its pages go back, it keeps its tokens (prompt and output), its
-state slot and its place at the front of the waiting queue, and is computed
-again from position 0 later; it samples again only when it has caught up
-(reference: qwen3_runtime/engine/scheduler.py:56-58,297-306). If nothing is
-running and the first waiting request still cannot get a page, that is an
-error. A request whose prompt plus ``max_tokens`` can never fit the pool or the
-position limit is refused when it is added
+When pages run out. A candidate whose offer comes to nothing is passed over for
+this step: a resident waits with its pages, a queued request keeps its place.
+If the whole walk yields nothing, the newest resident is sent back to the head
+of the queue: its pages return to the pool, it keeps its tokens (prompt and
+output so far) and its state slot, and will be computed again from position 0,
+sampling again only when it has caught up
+(reference: qwen3_runtime/engine/scheduler.py:56-58,297-306). With no resident
+left and the head of the queue still without a page the pool is held by
+someone else: an error. A request whose prompt plus ``max_tokens`` can never
+fit the pool or the position limit is refused on arrival
 (reference: qwen3_runtime/engine/scheduler.py:34-42).
 """
 
@@ -25,153 +29,127 @@ from collections import deque
 
 from ..cache import CacheManager
 from ..config.engine import EngineConfig
-from .request import Request, RequestStatus
+from .request import Phase, Request
 
 
 class Scheduler:
-    def __init__(self, config: EngineConfig, cache: CacheManager, max_model_len: int):
+    def __init__(self, config: EngineConfig, cache: CacheManager, max_model_len: int,
+                 portion_multiple: int = 1):
         self.config = config
         self.cache = cache
         self.max_model_len = int(max_model_len)
-        self.waiting: deque[Request] = deque()
-        self.running: deque[Request] = deque()
+        # a portion that does not end its request's tokens is a multiple of this many tokens
+        # (a mixer that works in blocks of its own asks for it; 1 for attention)
+        self.portion_multiple = max(1, int(portion_multiple))
+        self.queue: deque[Request] = deque()
+        self.residents: list[Request] = []
         self.num_preemptions = 0
 
-    # ---- queue ---------------------------------------------------------------
+    # ---- arrivals ------------------------------------------------------------------
     def add(self, req: Request) -> None:
-        max_len = len(req.token_ids) + req.max_tokens
+        longest = len(req.token_ids) + req.max_tokens
         # the last sampled token is never fed back, so it needs neither a page nor a position
-        if max_len - 1 > self.max_model_len:
+        if longest - 1 > self.max_model_len:
             raise RuntimeError(
-                f"request length {max_len} exceeds the model's limit of {self.max_model_len} positions"
-            )
-        needed = self.cache.pages_needed_for(max_len)
-        if self.cache.groups and needed > self.cache.num_pages:
+                f"request length {longest} exceeds the model's limit of {self.max_model_len} positions")
+        pages = self.cache.pages_needed_for(longest)
+        if self.cache.groups and pages > self.cache.num_pages:
             raise RuntimeError(
-                f"request length {max_len} needs {needed} cache pages; the pool has {self.cache.num_pages}"
-            )
-        req.status = RequestStatus.WAITING
-        self.waiting.append(req)
+                f"request length {longest} needs {pages} cache pages; the pool has {self.cache.num_pages}")
+        req.phase = Phase.QUEUED
+        self.queue.append(req)
 
     def is_finished(self) -> bool:
-        return not self.waiting and not self.running
+        return not self.queue and not self.residents
 
-    def computed(self, req: Request) -> int:
-        return self.cache.length(req.request_id) if req.admitted else 0
+    def behind(self, req: Request) -> int:
+        """Tokens of the request that are not in the cache yet."""
+        stored = self.cache.length(req.request_id) if req.holds_slot else 0
+        return len(req.token_ids) - stored
 
-    def uncomputed(self, req: Request) -> int:
-        return max(0, len(req.token_ids) - self.computed(req))
-
-    # ---- one step's decision ---------------------------------------------------
+    # ---- one step's decision ---------------------------------------------------------
     def schedule(self) -> list[Request]:
-        bound = self.config.max_num_seqs + len(self.running) + len(self.waiting) + 1
-        for _ in range(bound):
-            scheduled: list[Request] = []
-            budget = self._schedule_running(scheduled, self.config.max_num_batched_tokens)
-            self._schedule_waiting(scheduled, budget)
-            if scheduled:
-                return scheduled
-            if self.running:
-                self._preempt(self.running.pop())
-                continue
-            if self.waiting:
-                raise RuntimeError("the first waiting request cannot get a cache page although nothing is running")
-            return []
-        raise RuntimeError("scheduler could not form a step after preempting every request")
+        while True:
+            step = self._walk()
+            if step:
+                return step
+            if not self.residents:
+                if self.queue:
+                    raise RuntimeError(
+                        "the first waiting request cannot get a cache page although nothing is running")
+                return []
+            self._send_back(self.residents[-1])  # at most once per resident: the loop ends
 
-    def _portion(self, req: Request, budget: int) -> int:
-        remaining = self.uncomputed(req)
-        if remaining <= 0 or budget <= 0:
+    def _offer(self, req: Request, tokens_left: int) -> int:
+        want = min(self.behind(req), tokens_left)
+        if want <= 0:
             return 0
-        return self.cache.max_reservable_tokens(req.request_id, min(remaining, budget))
+        n = self.cache.max_reservable_tokens(req.request_id, want)
+        if n < self.behind(req) and self.portion_multiple > 1:
+            n -= n % self.portion_multiple
+        return max(0, n)
 
-    def _schedule_running(self, scheduled: list[Request], budget: int) -> int:
-        for req in self.running:
-            if len(scheduled) >= self.config.max_num_seqs or budget <= 0:
+    def _walk(self) -> list[Request]:
+        tokens_left, seats_left = self.config.max_num_batched_tokens, self.config.max_num_seqs
+        step: list[Request] = []
+        for req in self.residents + list(self.queue):
+            if tokens_left <= 0 or seats_left <= 0:
                 break
-            n = self._portion(req, budget)
-            if n <= 0:
-                continue  # no page for it now: it sits this step out
-            self.cache.reserve(req.request_id, n)
-            req.num_scheduled_tokens = n
-            scheduled.append(req)
-            budget -= n
-        return budget
-
-    def _schedule_waiting(self, scheduled: list[Request], budget: int) -> None:
-        deferred: list[Request] = []
-        while self.waiting:
-            if len(scheduled) >= self.config.max_num_seqs or budget <= 0:
-                break
-            req = self.waiting.popleft()
-            if not req.admitted:
+            if not req.holds_slot:
                 if self.cache.slots.num_free == 0:
-                    deferred.append(req)
-                    break  # later requests must not overtake it for a slot
+                    break  # nobody behind it in the queue may take the next free slot
                 self.cache.admit(req.request_id)
-                req.admitted = True
-            n = self._portion(req, budget)
-            if n <= 0:
-                deferred.append(req)
+                req.holds_slot = True
+            n = self._offer(req, tokens_left)
+            if n == 0:
                 continue
             self.cache.reserve(req.request_id, n)
-            req.num_scheduled_tokens = n
-            req.status = RequestStatus.RUNNING
-            scheduled.append(req)
-            self.running.append(req)
-            budget -= n
-        self.waiting.extendleft(reversed(deferred))
+            req.grant = n
+            tokens_left -= n
+            seats_left -= 1
+            step.append(req)
+        for req in step:
+            if req.phase is Phase.QUEUED:
+                self.queue.remove(req)
+                self.residents.append(req)
+                req.phase = Phase.RUNNING
+        return step
 
-    def _preempt(self, req: Request) -> None:
+    def _send_back(self, req: Request) -> None:
         self.cache.restart(req.request_id)
-        req.num_scheduled_tokens = 0
-        req.num_preemptions += 1
-        req.status = RequestStatus.WAITING
-        self.waiting.appendleft(req)
+        self.residents.remove(req)
+        self.queue.appendleft(req)
+        req.phase, req.grant = Phase.QUEUED, 0
+        req.restarts += 1
         self.num_preemptions += 1
 
-    # ---- after the step ----------------------------------------------------------
-    def postprocess(self, reqs: list[Request], token_ids: list[int | None]) -> list[Request]:
-        """The step's tokens are in the cache; append sampled tokens; finish what is done
-        (reference: qwen3_runtime/engine/scheduler.py:66-87)."""
-        if len(token_ids) != len(reqs):
-            raise ValueError("token_ids must align with scheduled requests")
-        finished = []
-        for req, tok in zip(reqs, token_ids):
-            req.num_scheduled_tokens = 0
-            if tok is None:
+    # ---- after the step ------------------------------------------------------------------
+    def settle(self, step: list[Request], sampled: list[int | None]) -> list[Request]:
+        """The step's tokens are in the cache. ``sampled[i]`` is the new token of ``step[i]``, or
+        None for a portion that did not reach the end of its request's tokens. Returns the
+        requests that ended (reference: qwen3_runtime/engine/scheduler.py:66-87)."""
+        if len(sampled) != len(step):
+            raise ValueError(f"{len(sampled)} sampled tokens for a step of {len(step)} requests")
+        ended = []
+        for req, token in zip(step, sampled):
+            req.grant = 0
+            if token is None:
                 continue
-            req.token_ids.append(int(tok))
-            reason = self._finish_reason(req)
+            reason = req.accept(token, self.config.eos_token_id)
             if reason is not None:
-                req.finish_reason = reason
-                self.finish(req)
-                finished.append(req)
-        return finished
+                self.retire(req, reason)
+                ended.append(req)
+        return ended
 
-    def _finish_reason(self, req: Request) -> str | None:
-        """Stop ids count only when ``ignore_eos`` is off and ``min_tokens`` are out; then length
-        (reference: qwen3_runtime/engine/scheduler.py:106-122)."""
-        n_out = req.num_output_tokens
-        tok = req.token_ids[-1]
-        hit_stop = (not req.ignore_eos) and (
-            tok in req.stop_token_ids
-            or (self.config.eos_token_id is not None and tok == self.config.eos_token_id)
-        )
-        if hit_stop and n_out >= req.min_tokens:
-            return "stop"
-        if n_out >= req.max_tokens:
-            return "length"
-        return None
-
-    def finish(self, req: Request) -> None:
-        """Give back pages and slot; also the way to cancel a request."""
-        req.status = RequestStatus.FINISHED
-        if req.admitted:
+    def retire(self, req: Request, reason: str) -> None:
+        """The request ends (also: is cancelled): pages and slot go back."""
+        if req.done:
+            return
+        if req in self.residents:
+            self.residents.remove(req)
+        elif req in self.queue:
+            self.queue.remove(req)
+        if req.holds_slot:
             self.cache.release(req.request_id)
-            req.admitted = False
-        for queue in (self.running, self.waiting):
-            try:
-                queue.remove(req)
-            except ValueError:
-                pass
+            req.holds_slot = False
+        req.phase, req.finish_reason = Phase.DONE, req.finish_reason or reason

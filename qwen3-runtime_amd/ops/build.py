@@ -1,8 +1,10 @@
 """Compile the HIP sources into shared libraries, in-tree, and find them again.
 
-Two kinds of library: ``core`` (everything whose sizes are run-time arguments)
-and ``attn_bf16_d<D>`` (the MFMA attention kernel, one build per head size).
-A library is rebuilt when the hash of its sources and flags changes. The build
+Two kinds of library of the engine's own: ``core`` (everything whose sizes are
+run-time arguments) and ``attn_bf16_d<D>`` (the MFMA attention kernel, one build
+per head size). A part defined elsewhere brings its kernels with
+``register_library(name, sources)`` and loads them with ``ops.hip.load_library``:
+same flags, same cache, same error reporting, no edit here. A library is rebuilt when the hash of its sources and flags changes. The build
 is plain ``hipcc`` for gfx950: seconds per file, no Python headers involved, so
 a fresh checkout compiles what a model needs at its first call and prints a
 line per file while it does.
@@ -36,6 +38,31 @@ class BuildError(RuntimeError):
     pass
 
 
+# libraries registered from outside: name -> (source paths, extra defines)
+_REGISTERED: dict[str, tuple[list[Path], list[str]]] = {}
+
+
+def register_library(name: str, sources, defines=()) -> None:
+    """Make ``name`` buildable and loadable: ``sources`` are paths of HIP files (they may
+    include ``common.h`` of this package, which is on the include path, and then link
+    ``runtime.hip`` for ``qrt_fail`` / ``qrt_last_error`` by listing it as ``"runtime.hip"``).
+    Registering the same name with the same sources again is allowed."""
+    if name == "core" or name.startswith("attn_bf16_d"):
+        raise BuildError(f"{name!r} is a library of the engine's own")
+    paths = [CSRC / s if not Path(s).is_absolute() else Path(s) for s in sources]
+    for path in paths:
+        if not path.is_file():
+            raise BuildError(f"library {name!r}: no source file {path}")
+    entry = (paths, list(defines))
+    if _REGISTERED.get(name, entry) != entry:
+        raise BuildError(f"library {name!r} is already registered with other sources")
+    _REGISTERED[name] = entry
+
+
+def registered_libraries() -> list[str]:
+    return sorted(_REGISTERED)
+
+
 def _say(msg: str) -> None:
     print(f"[qwen3_runtime_amd] {msg}", file=sys.stderr, flush=True)
 
@@ -67,24 +94,26 @@ def _hipcc() -> str:
     raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin)")
 
 
-def library_spec(name: str) -> tuple[list[str], list[str]]:
-    """Sources and extra defines of a library name."""
+def library_spec(name: str) -> tuple[list, list[str]]:
+    """Sources (names under ``csrc``, or paths) and extra defines of a library name."""
     if name == "core":
         return CORE_SOURCES, []
+    if name in _REGISTERED:
+        return list(_REGISTERED[name][0]), list(_REGISTERED[name][1])
     if name.startswith("attn_bf16_d"):
         d = int(name[len("attn_bf16_d"):])
         if d % 16 or not 16 <= d <= 512:
             raise BuildError(f"the bfloat16 attention kernel takes head sizes 16..512 in steps of 16, not {d}")
         return ["runtime.hip", "attention_bf16.hip"], [f"-DQRT_HEAD_DIM={d}"]
-    raise BuildError(f"unknown library {name!r}")
+    raise BuildError(f"unknown library {name!r}; registered from outside: {registered_libraries()}")
 
 
-def _digest(sources: list[str], defines: list[str]) -> str:
+def _digest(sources: list, defines: list[str]) -> str:
     h = hashlib.sha256()
     h.update(" ".join(FLAGS + defines).encode())
-    for name in sources + ["common.h"]:
-        h.update(name.encode())
-        h.update((CSRC / name).read_bytes())
+    for name in list(sources) + ["common.h"]:
+        h.update(Path(name).name.encode())
+        h.update((CSRC / name).read_bytes())  # an absolute path stays itself under "/"
     return h.hexdigest()
 
 
@@ -100,7 +129,7 @@ def is_current(name: str) -> bool:
 
 
 def _compile_one(hipcc: str, src: Path, obj: Path, defines: list[str]) -> None:
-    cmd = [hipcc, *FLAGS, *defines, "-c", str(src), "-o", str(obj)]
+    cmd = [hipcc, *FLAGS, *defines, f"-I{CSRC}", "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise BuildError(f"hipcc failed on {src.name}:\n{proc.stderr[-4000:]}")
@@ -122,12 +151,12 @@ def build_library(name: str, force: bool = False) -> Path:
         work.mkdir(exist_ok=True)
         t0 = time.time()
         _say(f"compiling {name} for {ARCH}: {len(sources)} files")
-        objs = [work / (Path(s).stem + ".o") for s in sources]
+        objs = [work / f"{i}_{Path(s).stem}.o" for i, s in enumerate(sources)]
 
         def one(pair):
             src, obj = pair
             _compile_one(hipcc, CSRC / src, obj, defines)
-            _say(f"  {src} done ({time.time() - t0:.0f} s)")
+            _say(f"  {Path(src).name} done ({time.time() - t0:.0f} s)")
 
         with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
             list(pool.map(one, zip(sources, objs)))
@@ -145,5 +174,5 @@ def build_library(name: str, force: bool = False) -> Path:
 
 def build_all(head_dims=(16, 32, 48, 64, 80, 96, 112, 128, 256), force: bool = True) -> list[Path]:
     """Every library the tests, the smoke run and the measurements load."""
-    names = ["core"] + [f"attn_bf16_d{d}" for d in head_dims]
+    names = ["core"] + [f"attn_bf16_d{d}" for d in head_dims] + registered_libraries()
     return [build_library(n, force=force) for n in names]

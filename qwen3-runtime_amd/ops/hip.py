@@ -84,7 +84,8 @@ def _load(name: str) -> ctypes.CDLL:
         lib = ctypes.CDLL(str(path))
     except OSError as exc:
         raise OpsError(f"cannot load {path}: {exc}") from exc
-    lib.qrt_last_error.restype = ctypes.c_char_p
+    if hasattr(lib, "qrt_last_error"):  # a library from outside need not link runtime.hip
+        lib.qrt_last_error.restype = ctypes.c_char_p
     return lib
 
 
@@ -103,6 +104,17 @@ def attention_library(head_dim: int) -> ctypes.CDLL:
     if head_dim not in _attn:
         _attn[head_dim] = _load(f"attn_bf16_d{head_dim}")
     return _attn[head_dim]
+
+
+_extra: dict[str, ctypes.CDLL] = {}
+
+
+def load_library(name: str) -> ctypes.CDLL:
+    """A library registered with ``ops.build.register_library``, built if need be, as a
+    ``ctypes.CDLL``; its entry points take raw device pointers and ``current_stream()``."""
+    if name not in _extra:
+        _extra[name] = _load(name)
+    return _extra[name]
 
 
 def _ptr(t: torch.Tensor | None):
@@ -127,6 +139,9 @@ def _stream() -> c_void_p:
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+current_stream = _stream
+
+
 def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> torch.Tensor:
     if not t.is_cuda:
         raise OpsError(f"{name} must be on the GPU, it is on {t.device}")
@@ -137,6 +152,9 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> torch.Tensor:
     if shape is not None and tuple(t.shape) != tuple(shape):
         raise OpsError(f"{name} must have shape {tuple(shape)}, it has {tuple(t.shape)}")
     return t
+
+
+check_tensor = _need  # for parts that call a library of their own
 
 
 class HipOps:
@@ -151,7 +169,7 @@ class HipOps:
     # from 12 rows on; a decode step is as fast either way at batch 8 and 5 % faster with it
     # at batch 16.
     shared_from_rows = {"whole": 17, "gated": 12, "planes": 9}
-    # tiles of 16 rows per wave in the attention kernel for long portions (1, 2 or 4)
+    # tiles of 16 rows per wave in the attention kernel for long portions (1 or 2)
     prefill_row_tiles = 2
     # long portions: keys and values go through LDS, shared by the four waves of a block
     prefill_through_lds = True
@@ -530,7 +548,9 @@ class HipOps:
         waves = 1 if max_rows <= 16 else (2 if max_rows <= 32 else 4)
         # long portions: several row tiles per wave, so that loaded keys and values serve more rows
         row_tiles = 1 if max_rows <= 64 else (self.prefill_row_tiles if d <= 128 else min(2, self.prefill_row_tiles))
-        key = ("attn_plan", g, decode, None if subset is None else tuple(subset))
+        # the list depends on the rows a tile holds (head geometry and kernel choice): layers of
+        # another geometry in the same step get a list of their own
+        key = ("attn_plan", g, nkv, d, waves, row_tiles, decode, None if subset is None else tuple(subset))
         plan = ctx.scratch.get(key)
         if plan is None:  # the same for every layer of the step
             dev = q.device

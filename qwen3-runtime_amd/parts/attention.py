@@ -83,15 +83,16 @@ class GroupedQueryAttention(Mixer):
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         qkv = ops.linear(x, self.qkv)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        inv_freq = getattr(self.position, "inv_freq", None)
-        if self.position is None or inv_freq is not None:
+        fused = self.position is None or self.position.fused_form == "neox_full"
+        if fused:
             # norm, rotation and the cache write in one pass over qkv
+            inv_freq = None if self.position is None else self.position.inv_freq
             q = ops.qk_norm_rope_store(
                 qkv, nq, nkv, d, self.q_norm, self.k_norm, eps, inv_freq, ctx.positions,
                 cache if cache.writes else None,
             )
         else:
-            # a position encoding this file does not know: norm, let it rotate, then store
+            # an encoding the fused kernel has no form for: norm, let it rotate, then store
             q, k, v = ops.qk_norm_split(qkv, nq, nkv, d, self.q_norm, self.k_norm, eps)
             q, k = self.position.rotate(ctx, q, k)
             if cache.writes:

@@ -41,6 +41,8 @@ class WeightFetcher(Protocol):
 
     def vector_f32(self, file_name: str) -> torch.Tensor: ...
 
+    def table_i32(self, file_name: str) -> torch.Tensor: ...
+
     def constant(self, tensor: torch.Tensor) -> torch.Tensor: ...
 
 
@@ -48,6 +50,13 @@ class Part:
     """Base of all parts: holds the tensor-name map, declares and loads tensors."""
 
     role = ""
+    # What the step function and the scheduler must know of a part, declared by its class:
+    # ``graph_capturable``: False for a part whose ``forward`` reads device memory on the host,
+    # or does anything else a captured HIP graph cannot replay; steps of a model with such a
+    # part run eagerly. ``portion_multiple``: a part that works on blocks of this many tokens
+    # wants every portion of a prompt but the last to be a multiple of it.
+    graph_capturable = True
+    portion_multiple = 1
 
     def __init__(self, tensors: Mapping[str, str] | None = None):
         self.tensor_names: dict[str, str] = dict(tensors or {})
@@ -88,6 +97,12 @@ class Norm(Part):
 
 class PositionEncoding(Part):
     role = "position"
+    # An encoding that the fused q/k kernel can apply itself says which of the kernel's forms
+    # it is; the attention mixer then never calls ``rotate``. The one form there is:
+    # ``"neox_full"``, the rotation of all ``head_dim`` elements, first half against second
+    # half, by the angles ``position * self.inv_freq[j]`` (float32 [head_dim / 2] on the device).
+    # None (the default) means the mixer norms, calls ``rotate`` and stores, as three steps.
+    fused_form: str | None = None
 
 
 class Block(Part):

@@ -7,6 +7,7 @@ fixed loop: qwen3_runtime/models/qwen3.py:222-266).
 
 from __future__ import annotations
 
+import math
 from typing import Sequence
 
 from ..registry import part_class
@@ -63,6 +64,16 @@ class DecoderModel:
             yield from walk(block)
         yield from walk(self.final_norm)
         yield from walk(self.head)
+
+    @property
+    def graph_capturable(self) -> bool:
+        """Whether a step of this model may be captured into a HIP graph: every part says so."""
+        return all(part.graph_capturable for part in self.parts())
+
+    @property
+    def portion_multiple(self) -> int:
+        """Least common multiple of what the parts ask of a prompt's portions."""
+        return math.lcm(*(max(1, int(part.portion_multiple)) for part in self.parts()))
 
     def tensor_decls(self) -> list[TensorDecl]:
         """Every tensor the model reads, once per file name."""

@@ -34,11 +34,15 @@ class TensorDecl:
 
     ``init`` tells the random-weights mode how to draw it: ``"matrix"`` and
     ``"embedding"`` are zero-mean normal, ``"norm"`` is a scale around one.
+    ``storage`` is ``"float"`` (stored as bfloat16, float32 or float16) or ``"int"``
+    (an integer table, held as int32; drawn as zeros in the random-weights mode unless
+    ``init`` is ``"index:<n>"``, uniform in ``[0, n)``).
     """
 
     file_name: str
     shape: tuple[int, ...]
     init: str = "matrix"
+    storage: str = "float"
 
 
 @dataclass(frozen=True)

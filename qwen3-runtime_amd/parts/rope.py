@@ -17,6 +17,8 @@ from .base import PositionEncoding
 
 @register_part("position", "rope_neox")
 class RotaryNeox(PositionEncoding):
+    fused_form = "neox_full"
+
     def __init__(self, head_dim: int, theta: float, tensors=None):
         super().__init__(tensors)
         if head_dim % 2:

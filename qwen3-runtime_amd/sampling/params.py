@@ -28,26 +28,26 @@ class SamplingParams:
     logprobs: bool = False
 
     def __post_init__(self) -> None:
-        if not math.isfinite(self.temperature):
-            raise ValueError("temperature must be finite")
-        if not math.isfinite(self.top_p) or not 0.0 < self.top_p <= 1.0:
-            raise ValueError("top_p must satisfy 0 < top_p <= 1")
-        if not math.isfinite(self.min_p) or not 0.0 <= self.min_p <= 1.0:
-            raise ValueError("min_p must satisfy 0 <= min_p <= 1")
+        def finite(name: str) -> float:
+            value = float(getattr(self, name))
+            if not math.isfinite(value):
+                raise ValueError(f"{name} is {value}; it has to be a finite number")
+            return value
+
+        finite("temperature")
+        if not 0.0 < finite("top_p") <= 1.0:
+            raise ValueError(f"top_p is {self.top_p}; it is a probability mass in (0, 1]")
+        if not 0.0 <= finite("min_p") <= 1.0:
+            raise ValueError(f"min_p is {self.min_p}; it is a share of the largest probability, in [0, 1]")
+        if finite("repetition_penalty") <= 0.0:
+            raise ValueError(f"repetition_penalty is {self.repetition_penalty}; logits are divided by it, so it is > 0")
+        finite("presence_penalty")
+        finite("frequency_penalty")
         if self.min_tokens < 0:
-            raise ValueError("min_tokens must be non-negative")
-        if self.repetition_penalty <= 0 or not math.isfinite(self.repetition_penalty):
-            raise ValueError("repetition_penalty must be positive and finite")
-        for name in ("presence_penalty", "frequency_penalty"):
-            if not math.isfinite(getattr(self, name)):
-                raise ValueError(f"{name} must be finite")
+            raise ValueError(f"min_tokens is {self.min_tokens}; a count of tokens cannot be negative")
 
     def is_greedy(self) -> bool:
         return self.temperature <= 0.0
 
     def has_penalties(self) -> bool:
-        return not (
-            self.repetition_penalty == 1.0
-            and self.presence_penalty == 0.0
-            and self.frequency_penalty == 0.0
-        )
+        return (self.repetition_penalty, self.presence_penalty, self.frequency_penalty) != (1.0, 0.0, 0.0)

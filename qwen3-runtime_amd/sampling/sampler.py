@@ -54,7 +54,7 @@ class Sampler:
             toks = torch.tensor([int(b[1]) for b in bias], dtype=torch.int32, device=self.device)
             vals = torch.tensor([float(b[2]) for b in bias], dtype=torch.float32, device=self.device)
             self.ops.add_bias(logits, rows, toks, vals)
-        forced = [r.next_forced_token() for r in reqs]
+        forced = [r.forced_next() for r in reqs]
         any_forced = any(f is not None for f in forced)
         tok, lp, work, both = self.ops.sample(logits, slot_rows, self.fparams, self.iparams, self.seeds,
                                               self.counts, keep_processed=any_forced)

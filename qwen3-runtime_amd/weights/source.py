@@ -75,7 +75,8 @@ class RandomSource:
     values do not depend on which other tensors exist or on the order they are
     asked for. ``"matrix"`` and ``"embedding"`` tensors are N(0, std);
     ``"norm"`` tensors are ``1 + N(0, norm_jitter)`` (all ones when the jitter
-    is zero). Values are rounded to ``store_dtype``.
+    is zero). Values are rounded to ``store_dtype``. Integer tables
+    (``storage="int"``) are int32: zeros, or uniform in ``[0, n)`` for ``init="index:<n>"``.
     """
 
     def __init__(
@@ -102,13 +103,18 @@ class RandomSource:
         return tuple(self._decls[name].shape)
 
     def dtype(self, name: str) -> torch.dtype:
-        return self.store_dtype
+        return torch.int32 if self._decls[name].storage == "int" else self.store_dtype
 
     def get(self, name: str, device: torch.device | str = "cpu") -> torch.Tensor:
         decl = self._decls[name]
         digest = hashlib.sha256(f"{self.seed}:{name}".encode()).digest()
         gen = torch.Generator(device=device)
         gen.manual_seed(int.from_bytes(digest[:8], "little") & (2**63 - 1))
+        if decl.storage == "int":
+            if decl.init.startswith("index:"):
+                return torch.randint(0, int(decl.init[6:]), decl.shape, generator=gen, dtype=torch.int32,
+                                     device=device)
+            return torch.zeros(decl.shape, dtype=torch.int32, device=device)
         x = torch.randn(decl.shape, generator=gen, dtype=torch.float32, device=device)
         if decl.init == "norm":
             x = 1.0 + self.norm_jitter * x
@@ -144,7 +150,7 @@ def write_model_folder(
     tensors = {}
     for decl in decls:
         t = source.get(decl.file_name)
-        keep_f32 = decl.file_name in f32_names
+        keep_f32 = decl.file_name in f32_names or decl.storage == "int"  # integers stay int32
         # round through the storage type so that every reader sees equal values
         tensors[decl.file_name] = (t if keep_f32 else t.to(store_dtype)).contiguous()
     folder = Path(folder)

@@ -1,7 +1,7 @@
 """Plain, slow Qwen3 dense decoder: whole sequences, no cache, one function per part.
 
-Written from the reference's formulas; every function cites where the formula
-stands in /root/reference. It shares no code with the engine: it parses
+Written from the reference's formulas; every function cites the file and lines of
+yuzheng310/qwen3-runtime where its formula stands. It shares no code with the engine: it parses
 config.json and reads the safetensors file itself. Arithmetic runs in float64
 unless ``dtype`` says otherwise, except rotation angles, which the reference
 fixes to float32 (the table is built in float32).

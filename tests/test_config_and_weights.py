@@ -137,6 +137,44 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert piece in text
 
 
+def test_an_integer_tensor_where_a_matrix_is_read_is_an_error(tmp_path):
+    """A tensor of the right name and shape but stored as integers (a quantised file, say) must
+    not be cast silently into weights; it is named in the same single error."""
+    from safetensors.torch import load_file, save_file
+
+    cfg = preset("tiny_a")
+    folder = write_model_folder(tmp_path / "m", cfg.to_dict(), seed=1)
+    tensors = load_file(str(folder / "model.safetensors"))
+    name = "model.layers.1.self_attn.q_proj.weight"
+    tensors[name] = torch.zeros(tensors[name].shape, dtype=torch.int8)
+    del tensors["model.norm.weight"]
+    save_file(tensors, str(folder / "model.safetensors"))
+    with pytest.raises(WeightError) as err:
+        load_model(model_of(cfg), SafetensorsSource(folder), "cpu", torch.float32)
+    assert err.value.wrong_dtype == [(name, "int8", "bfloat16, float32 or float16")]
+    assert err.value.missing == ["model.norm.weight"]
+    assert "wrong types (1)" in str(err.value) and "stored as int8" in str(err.value)
+
+
+def test_integer_tables_are_declared_drawn_and_kept_as_int32():
+    """A part may declare an integer table: it is drawn as integers, stored as int32, loaded
+    as int32 in both engine types, and a floating tensor in its place is an error."""
+    from qwen3_runtime_amd.parts.plan import TensorDecl
+    from qwen3_runtime_amd.weights.loader import WeightLoader
+
+    decls = [TensorDecl("perm", (7,), init="index:5", storage="int"), TensorDecl("w", (3, 4))]
+    src = RandomSource(decls, 3)
+    assert src.dtype("perm") == torch.int32 and src.dtype("w") == torch.bfloat16
+    perm = src.get("perm")
+    assert perm.dtype == torch.int32 and 0 <= int(perm.min()) and int(perm.max()) < 5
+    check_source(src, decls)
+    for engine_dtype in (torch.bfloat16, torch.float32):
+        assert WeightLoader(src, "cpu", engine_dtype).table_i32("perm").dtype == torch.int32
+    swapped = RandomSource([TensorDecl("perm", (7,)), TensorDecl("w", (3, 4))], 3)
+    with pytest.raises(WeightError, match="perm is stored as bfloat16, expected an integer type"):
+        check_source(swapped, decls)
+
+
 def test_tied_model_may_carry_an_unused_head(tmp_path):
     from safetensors.torch import load_file, save_file
 

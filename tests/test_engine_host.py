@@ -97,3 +97,62 @@ def test_which_kernel_multiplies_how_many_rows():
     assert seqs[0] == 1                  # the tile that sees 900 keys goes first
     sub, n_sub = HipOps.plan_tiles([70, 33], [200, 33], g, 64, nkv=2, seq_ids=[0, 2])
     assert sorted(set(sub[:n_sub].tolist())) == [0, 2]
+
+
+def cpu_engine(folder, page_size, num_pages):
+    from qwen3_runtime_amd.llm import build_engine
+
+    return build_engine(folder, block_size=page_size, num_kv_blocks=num_pages, max_num_seqs=2, dtype="float32",
+                        device="cpu", cuda_graph=False, ops=TorchOps())
+
+
+def test_ids_that_would_index_device_memory_are_checked_on_arrival(model_folders, tiny_configs):
+    """Prompt ids, forced ids and logit_bias keys all end up as indices in kernels (embedding
+    rows, columns of the logits, penalty counts): one outside the vocabulary is refused when the
+    request is added, with nothing queued."""
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    cfg, page = tiny_configs["tiny_a"]
+    eng = cpu_engine(model_folders["tiny_a"], page, 8)
+    v = cfg.vocab_size
+    with pytest.raises(ValueError, match="prompt token"):
+        eng.add_request([1, v])
+    with pytest.raises(ValueError, match="prompt token"):
+        eng.add_request([-1])
+    with pytest.raises(ValueError, match=f"forced token {v + 5}"):
+        eng.add_request([1, 2], forced_tokens=[3, v + 5])
+    with pytest.raises(ValueError, match="logit_bias key -2"):
+        eng.add_request([1, 2], sampling=SamplingParams(logit_bias={-2: 1.0}))
+    with pytest.raises(ValueError, match=f"logit_bias key {v}"):
+        eng.add_request([1, 2], sampling=SamplingParams(logit_bias={0: 1.0, v: 1.0}))
+    for bad in (float("nan"), float("inf")):
+        with pytest.raises(ValueError, match="a bias is a finite number"):
+            eng.add_request([1, 2], sampling=SamplingParams(logit_bias={3: bad}))
+    assert eng.is_finished() and not eng._live
+    # in range, and -inf (an excluded id), are taken
+    eng.add_request([1, v - 1], forced_tokens=[0, v - 1], sampling=SamplingParams(logit_bias={v - 1: float("-inf")}))
+    assert not eng.is_finished()
+
+
+def test_default_page_count_is_capped_by_what_requests_can_use(monkeypatch, model_folders):
+    """No page count given: the pool is sized from free memory but never beyond
+    max_num_seqs requests of max_model_len tokens (plus a spare page each)."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.config.model import read_config_json
+    from qwen3_runtime_amd.engine import factory
+
+    _, model = factory.build_model(read_config_json(model_folders["tiny_b"]))
+    per_page = 2 * 3 * 2 * 32 * 8 * 2          # keys and values, 3 layers, 2 heads of 32, 8 tokens, bfloat16
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (200 * 2**30, 288 * 2**30))
+    cfg = EngineConfig(page_size=8, max_num_seqs=4, max_model_len=100, dtype="bfloat16")
+    assert factory.pages_for_memory(model, cfg, torch.bfloat16, "cuda:0") == 4 * (13 + 1)
+    # memory is the limit when it is the smaller one; never fewer than 32 pages
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (40 * per_page, 288 * 2**30))
+    assert factory.pages_for_memory(model, cfg, torch.bfloat16, "cuda:0") == int(40 * 0.85)
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (per_page, 288 * 2**30))
+    assert factory.pages_for_memory(model, cfg, torch.bfloat16, "cuda:0") == 32
+    # without max_model_len the model's position limit stands in
+    cfg = EngineConfig(page_size=8, max_num_seqs=2, dtype="bfloat16")
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (200 * 2**30, 288 * 2**30))
+    limit = model.plan.max_positions
+    assert factory.pages_for_memory(model, cfg, torch.bfloat16, "cuda:0") == 2 * (-(-limit // 8) + 1)

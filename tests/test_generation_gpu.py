@@ -236,7 +236,7 @@ class _Req:
     def __init__(self, p):
         self.sampling = p
 
-    def next_forced_token(self):
+    def forced_next(self):
         return None
 
 
@@ -363,3 +363,114 @@ def test_logit_bias_and_penalty_counts_follow_the_output(model_folders):
         want.append(P.greedy(logits))
         ids.append(want[-1])
     assert out == want
+
+
+def test_engine_without_a_page_count(model_folders):
+    """``LLM(folder)`` as the README shows it, no ``num_kv_blocks``: the pool is sized from free
+    memory, capped by what max_num_seqs requests of the model's position limit can use (a tiny
+    model must not claim the device). Generates; every page and slot comes back."""
+    from qwen3_runtime_amd.llm import LLM
+
+    cfg, w = P.read_model(model_folders["tiny_b"])
+    free_before, _ = torch.cuda.mem_get_info()
+    m = LLM(str(model_folders["tiny_b"]), dtype="bfloat16", block_size=8)
+    cache = m.engine.cache
+    limit = cfg["max_position_embeddings"]
+    assert 32 <= cache.num_pages <= 4 * (-(-limit // 8) + 1)
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_before - free_after < 2**30, "a tiny model's cache took more than a GiB"
+    prompts = prompts_for(cfg, [12, 30], seed=2)
+    outs = m.generate(prompts, max_tokens=6)
+    assert [len(o) for o in outs] == [6, 6]
+    assert outs[0][0] == P.greedy_generate(cfg, w, prompts[0], 1)[0]
+    cache.check()
+    assert cache.num_free_pages == cache.num_pages and cache.slots.num_free == 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_command_line(model_folders, dtype):
+    """``python -m qwen3_runtime_amd.cli --model DIR`` as a user runs it, with no page count:
+    the ``runtime [...]`` line holds the plain implementation's greedy tokens
+    (reference, for the lines it prints: qwen3_runtime/reference/cli.py:51-56)."""
+    import ast
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    cfg, w = P.read_model(model_folders["tiny_a"])
+    prompt = [5, 17, 3, 250, 9]
+    proc = subprocess.run(
+        [sys.executable, "-m", "qwen3_runtime_amd.cli", "--model", str(model_folders["tiny_a"]), "--dtype", dtype,
+         "--prompt-tokens", *map(str, prompt), "--max-tokens", "6"],
+        capture_output=True, text=True, timeout=600, cwd=str(root))
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = dict(l.split(" ", 1) for l in proc.stdout.splitlines() if " " in l)
+    got = ast.literal_eval(lines["runtime"])
+    want = P.greedy_generate(cfg, w, prompt, 6)
+    assert got == want if dtype == "float32" else got[0] == want[0]
+    assert lines["bytes_per_block"] == str(2 * 2 * 2 * 16 * 16 * (4 if dtype == "float32" else 2))
+    assert lines["device"] == "cuda:0" and lines["backend"] == "hip" and lines["cuda_graph"] == "True"
+
+
+def test_graph_buffer_is_repacked_when_a_request_id_comes_back(model_folders):
+    """A decode graph keeps the packed block tables of its last step and, when the same request
+    ids come one token further, only patches them. A request that was released and admitted again
+    under the same id (or restarted after a preemption) owns other pages by then: the kept tables
+    must not be trusted. Same id, same length as the graph last saw plus one, other pages."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.batch import StepEntry
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg, _ = P.read_model(model_folders["tiny_b"])
+    ids = prompts_for(cfg, [40], seed=11)[0]
+    other = prompts_for(cfg, [40], seed=12)[0]
+
+    def run(graph):
+        engine_cfg = EngineConfig(page_size=8, num_pages=10, max_num_seqs=2, dtype="float32", device=DEV,
+                                  hip_graph=graph)
+        loaded = load(model_folders["tiny_b"], engine_cfg)
+        runner, cache = loaded.runner, loaded.cache
+        out = []
+        cache.admit("a")
+        runner.step([StepEntry("a", ids[:30], [])])
+        for p in range(30, 34):                      # eager, capture, replays
+            out.append(runner.step([StepEntry("a", ids[p: p + 1], [0])])[0].cpu().clone())
+        old_pages = list(cache.block_table(0, "a"))
+        cache.release("a")
+        cache.admit("a")                             # the same id again: the pool hands it other pages
+        runner.step([StepEntry("a", ids[:34], [])])  # up to the length the graph saw last
+        assert not set(cache.block_table(0, "a")) & set(old_pages)
+        cache.admit("squatter")                      # takes the pages "a" held before, and fills them
+        runner.step([StepEntry("squatter", other[:36], [])])
+        assert set(cache.block_table(0, "squatter")) == set(old_pages)
+        for p in range(34, 38):
+            out.append(runner.step([StepEntry("a", ids[p: p + 1], [0])])[0].cpu().clone())
+        return torch.stack(out), bool(runner._graphs)
+
+    eager, _ = run(False)
+    replayed, used = run(True)
+    assert used, "no decode step was replayed from a graph"
+    torch.testing.assert_close(replayed, eager, atol=2e-5, rtol=2e-5)
+    _, w = P.read_model(model_folders["tiny_b"])
+    want = P.forward(cfg, w, ids[:38])
+    torch.testing.assert_close(replayed, torch.cat([want[30:34], want[34:38]]).float(), atol=5e-5, rtol=5e-5)
+
+
+def test_sampler_with_an_excluded_id():
+    """A bias of -inf excludes an id: the row's first value being -inf must not poison the sum
+    of exponentials (greedy log-probability) nor be drawn."""
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    x = torch.tensor([[2.0, 1.0, 0.5, -1.0] * 64, [0.0, 3.0, 1.0, 2.0] * 64], device=DEV)
+    ban = {0: float("-inf"), 4: float("-inf")}
+    params = [(SamplingParams(logit_bias=ban), 0), (SamplingParams(temperature=1.0, seed=5, logit_bias={1: float("-inf")}), 5)]
+    s, rows = sample_rows(x, params)
+    tok, lp = s.sample(x, rows, [_Req(p) for p, _ in params])
+    biased = x.clone().cpu()
+    biased[0, [0, 4]] = float("-inf")
+    biased[1, 1] = float("-inf")
+    assert tok[0] == int(biased[0].argmax()) == 8
+    assert lp[0] == pytest.approx(float(torch.log_softmax(biased[0], -1)[8]), abs=1e-5)
+    assert tok[1] != 1 and math.isfinite(lp[1])
+    assert lp[1] == pytest.approx(float(torch.log_softmax(biased[1], -1)[tok[1]]), abs=1e-4)

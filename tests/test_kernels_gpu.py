@@ -359,6 +359,8 @@ ATTN_CASES = [
     ([(1, 100), (2, 61), (1, 24)], 4, 2, 32, 24),   # page sizes that are no power of two
     ([(20, 131), (300, 300)], 4, 1, 64, 40),
     ([(150, 210)], 2, 1, 256, 16),                  # a long portion at a head size whose LDS stages do not fit
+    ([(1, 333), (1, 40), (2, 700)], 4, 1, 256, 16),  # the decode kernel at head size 256 (more LDS than the default)
+    ([(1, 1500), (90, 90)], 4, 2, 256, 16),          # ... and beside a portion: two launches
 ]
 
 

@@ -17,23 +17,7 @@ pytestmark = pytest.mark.gpu
 TOL_F32 = dict(atol=2e-4, rtol=2e-4)
 
 
-def check_rounding_noise(got, want):
-    """bfloat16 against the float32 plain implementation. Activations are rounded to 8 bits of
-    mantissa some seven times per layer, which leaves an error that behaves like noise: measured
-    at both sizes and under every cutting, its root mean square is 1.0 % of the logits' standard
-    deviation and its largest value five times that (what 400,000 Gaussian samples give). The
-    bounds leave half as much again; a fault in a page, a mask or a portion's edge moves logits
-    by a sizeable part of their standard deviation."""
-    keys = sorted(want)
-    assert set(got) == set(want)
-    w = torch.stack([want[k].double() for k in keys])
-    err = torch.stack([got[k].double() for k in keys]) - w
-    std = float(w.std())
-    rms = float(err.pow(2).mean().sqrt())
-    worst = float(err.abs().max())
-    where = keys[int(err.abs().amax(dim=1).argmax())]
-    assert rms < 0.015 * std, f"rms error {rms:.4f} against a logit deviation of {std:.3f}"
-    assert worst < 0.08 * std, f"largest error {worst:.4f} at (request, position) {where}; logit deviation {std:.3f}"
+check_rounding_noise = traces.compare_rounding_noise
 
 
 @pytest.fixture(scope="module")

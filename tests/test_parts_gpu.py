@@ -6,6 +6,7 @@ reads another step's cache. It is stepped under every cutting and compared with 
 whole-sequence computation written out below."""
 
 import math
+from pathlib import Path
 
 import pytest
 import torch
@@ -15,6 +16,7 @@ from plain import qwen3_plain as P
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+TOY_KERNELS = Path(__file__).resolve().parent / "toy_ops.hip"
 
 
 class DictFetch:
@@ -147,7 +149,12 @@ def register_toy():
 
     @register_part("mixer", "toy_ema")
     class EmaMixer(Mixer):
-        """state <- decay * state + x_t;  y_t = gain * state.  One float32 vector per request."""
+        """state <- decay * state + x_t;  y_t = gain * state.  One float32 vector per request.
+        It reads the slots on the host, which a captured graph cannot replay, and says so; and it
+        asks for portions of a multiple of four tokens, as a mixer with blocks of its own would."""
+
+        graph_capturable = False
+        portion_multiple = 4
 
         def __init__(self, hidden_size, decay, tensors=None):
             super().__init__(tensors)
@@ -176,15 +183,33 @@ def register_toy():
 
     @register_part("position", "toy_scale")
     class ScalePosition(PositionEncoding):
-        """q and k are scaled by 1 + rate * position: not a rotation, and not fused with anything."""
+        """q and k are scaled by 1 + rate * position: not a rotation, not fused with anything, and
+        computed by a kernel of its own, which the part brings along as a library."""
 
         def __init__(self, rate, tensors=None):
+            from qwen3_runtime_amd.ops import build
+
             super().__init__(tensors)
             self.rate = rate
+            build.register_library("toy_ops", ["runtime.hip", TOY_KERNELS])
 
         def rotate(self, ctx, q, k):
-            f = (1.0 + self.rate * ctx.positions.float())[:, None, None]
-            return (q.float() * f).to(q.dtype), (k.float() * f).to(k.dtype)
+            from ctypes import c_float, c_int, c_void_p
+
+            from qwen3_runtime_amd.ops import hip
+
+            lib = hip.load_library("toy_ops")
+            out = []
+            for x in (q, k):
+                hip.check_tensor(x, "toy_scale input")
+                y = torch.empty_like(x)
+                code = lib.toy_scale_by_position(
+                    c_void_p(x.data_ptr()), c_void_p(y.data_ptr()), c_void_p(ctx.positions.data_ptr()),
+                    c_float(self.rate), c_int(x.shape[0]), c_int(x.shape[1] * x.shape[2]),
+                    c_int(0 if x.dtype == torch.float32 else 1), hip.current_stream())
+                assert code == 0, lib.qrt_last_error().decode()
+                out.append(y)
+            return tuple(out)
 
     @register_part("feed_forward", "toy_routed")
     class RoutedFeedForward(FeedForward):
@@ -393,3 +418,47 @@ def test_window_layer_gives_pages_back_while_decoding(toy_folder):
     torch.testing.assert_close(torch.stack(got), want[59:].float(), atol=5e-5, rtol=5e-5)
     cache.release("r")
     cache.check()
+
+
+def test_toy_architecture_with_graphs_asked_for(toy_folder):
+    """HIP graphs are asked for, but the toy's state mixer declares that it cannot be captured:
+    the runner then steps eagerly, with no change to the package, and the logits are right."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    reqs = traces.make_requests(TOY["vocab_size"], [45], seed=3)
+    steps = traces.tail_one_by_one(reqs, tail=20)
+    cfg = EngineConfig(page_size=8, num_pages=8, max_num_seqs=2, dtype="float32", device=DEV, hip_graph=True)
+    loaded = load(toy_folder, cfg)
+    assert not loaded.model.graph_capturable and not loaded.runner.hip_graph
+    got = traces.replay(loaded, steps)
+    logits = toy_plain(toy_folder, reqs["r0"])
+    traces.compare(got, {("r0", p): logits[p].float() for p in range(45)}, atol=5e-5, rtol=5e-5)
+
+
+def test_toy_architecture_generates_through_the_engine_in_portions_it_asked_for(toy_folder):
+    """Through scheduler and sampler: the toy's mixer wants portions of a multiple of four tokens,
+    the token limit is 10, so prompts advance by 8 until their last portion; greedy tokens equal
+    the whole-sequence computation's."""
+    from qwen3_runtime_amd.llm import build_engine
+
+    eng = build_engine(str(toy_folder), block_size=8, num_kv_blocks=24, max_num_seqs=2, max_num_batched_tokens=10,
+                       dtype="float32", device=DEV, cuda_graph=True)
+    assert eng.scheduler.portion_multiple == 4
+    prompts = list(traces.make_requests(TOY["vocab_size"], [23, 9], seed=4).values())
+    inner, log = eng.scheduler.schedule, []
+
+    def spy():
+        batch = inner()
+        log.extend((r.grant, eng.scheduler.behind(r)) for r in batch)  # before the step: what it gets, what it lacks
+        return batch
+
+    eng.scheduler.schedule = spy
+    outs = eng.generate_batch(prompts, max_tokens=5)
+    cut = [g for g, lacking in log if g < lacking]
+    assert cut and all(g % 4 == 0 for g in cut), log
+    for p, out in zip(prompts, outs):
+        ids = list(p)
+        for _ in range(5):
+            ids.append(int(toy_plain(toy_folder, ids)[-1].argmax()))
+        assert out == ids[len(p):]

@@ -6,7 +6,7 @@ import torch
 
 from qwen3_runtime_amd.cache import CacheManager
 from qwen3_runtime_amd.config.engine import EngineConfig
-from qwen3_runtime_amd.engine.request import Request, RequestStatus
+from qwen3_runtime_amd.engine.request import Phase, Request
 from qwen3_runtime_amd.engine.scheduler import Scheduler
 from qwen3_runtime_amd.parts.plan import CacheSpec
 from qwen3_runtime_amd.sampling.params import SamplingParams
@@ -21,10 +21,10 @@ def scheduler(num_pages=64, page_size=16, max_seqs=4, budget=512, eos=None, max_
 
 
 def run(s, batch, tokens):
-    """What the engine does between schedule() and postprocess(): the tokens are stored."""
+    """What the engine does between schedule() and settle(): the tokens are stored."""
     for r in batch:
-        s.cache.commit(r.request_id, r.num_scheduled_tokens)
-    return s.postprocess(batch, tokens)
+        s.cache.commit(r.request_id, r.grant)
+    return s.settle(batch, tokens)
 
 
 def test_first_portion_reserves_only_its_pages():
@@ -32,9 +32,9 @@ def test_first_portion_reserves_only_its_pages():
     req = Request(list(range(8192)), max_tokens=1)
     s.add(req)
     batch = s.schedule()
-    assert batch == [req] and req.num_scheduled_tokens == 512
+    assert batch == [req] and req.grant == 512
     assert len(s.cache.block_table(0, req.request_id)) == 32 and s.cache.num_free_pages == 481
-    assert req.status == RequestStatus.RUNNING
+    assert req.phase == Phase.RUNNING
 
 
 def test_budget_cuts_a_prompt_into_portions():
@@ -44,10 +44,10 @@ def test_budget_cuts_a_prompt_into_portions():
     sizes = []
     for _ in range(3):
         batch = s.schedule()
-        sizes.append(req.num_scheduled_tokens)
+        sizes.append(req.grant)
         run(s, batch, [None if sum(sizes) < 300 else 5])
     assert sizes == [128, 128, 44]
-    assert req.status == RequestStatus.FINISHED and req.finish_reason == "length"
+    assert req.phase == Phase.DONE and req.finish_reason == "length"
     assert s.cache.num_free_pages == 256
 
 
@@ -56,7 +56,7 @@ def test_two_prompts_share_the_budget():
     a, b = Request(list(range(8)), 1), Request(list(range(8, 16)), 1)
     s.add(a), s.add(b)
     assert s.schedule() == [a, b]
-    assert (a.num_scheduled_tokens, b.num_scheduled_tokens) == (8, 2)
+    assert (a.grant, b.grant) == (8, 2)
 
 
 def test_a_long_prompt_takes_the_whole_budget():
@@ -65,7 +65,7 @@ def test_a_long_prompt_takes_the_whole_budget():
     s.add(long), s.add(short)
     for _ in range(2):
         batch = s.schedule()
-        assert batch == [long] and long.num_scheduled_tokens == 2048
+        assert batch == [long] and long.grant == 2048
         run(s, batch, [None])
 
 
@@ -77,7 +77,7 @@ def test_decode_and_a_new_prompt_in_one_step():
     p = Request(list(range(40)), max_tokens=1)
     s.add(p)
     batch = s.schedule()
-    assert batch == [d, p] and (d.num_scheduled_tokens, p.num_scheduled_tokens) == (1, 15)
+    assert batch == [d, p] and (d.grant, p.grant) == (1, 15)
 
 
 def test_portion_shrinks_to_the_free_pages():
@@ -85,7 +85,7 @@ def test_portion_shrinks_to_the_free_pages():
     a, b = Request(list(range(31)), 1), Request(list(range(40)), 1)
     s.add(a), s.add(b)
     assert s.schedule() == [a, b]
-    assert (a.num_scheduled_tokens, b.num_scheduled_tokens) == (31, 32)
+    assert (a.grant, b.grant) == (31, 32)
     assert len(s.cache.block_table(0, b.request_id)) == 2
 
 
@@ -95,11 +95,11 @@ def test_throughput_shape_two_waves_then_mixed():
     for r in reqs:
         s.add(r)
     first = s.schedule()
-    assert len(first) == 8 and sum(r.num_scheduled_tokens for r in first) == 2048
+    assert len(first) == 8 and sum(r.grant for r in first) == 2048
     run(s, first, [1] * 8)
     second = s.schedule()
-    assert sum(1 for r in second if r.num_scheduled_tokens == 1) == 8
-    assert sum(r.num_scheduled_tokens for r in second) == 2048
+    assert sum(1 for r in second if r.grant == 1) == 8
+    assert sum(r.grant for r in second) == 2048
 
 
 def test_request_that_can_never_fit_is_refused():
@@ -119,12 +119,12 @@ def test_pages_run_out_the_youngest_is_preempted_and_recomputed():
     run(s, s.schedule(), [11, 22])
     assert s.cache.num_free_pages == 0
     batch = s.schedule()                      # both want a fifth page; none is free
-    assert s.num_preemptions == 1 and b.num_preemptions == 1
+    assert s.num_preemptions == 1 and b.restarts == 1
     # a decodes with one of the two freed pages; b restarts at once with the other
     # (reference: tests/cpu/test_scheduler.py:115-131 expects a restarted request in this batch)
-    assert batch == [a, b] and (a.num_scheduled_tokens, b.num_scheduled_tokens) == (1, 4)
+    assert batch == [a, b] and (a.grant, b.grant) == (1, 4)
     assert b.token_ids == list(range(8, 16)) + [22]          # keeps prompt and output
-    assert b.admitted                                          # keeps its slot
+    assert b.holds_slot                                          # keeps its slot
     slot = s.cache.slots.slot(b.request_id)
     run(s, batch, [12, None])
     # b comes back: recomputes prompt + its one token in portions, samples only when caught up
@@ -133,10 +133,10 @@ def test_pages_run_out_the_youngest_is_preempted_and_recomputed():
         batch = s.schedule()
         toks = []
         for r in batch:
-            end = s.cache.length(r.request_id) + r.num_scheduled_tokens
+            end = s.cache.length(r.request_id) + r.grant
             toks.append(7 if end >= len(r.token_ids) else None)
             if r is b:
-                seen.append((r.num_scheduled_tokens, toks[-1]))
+                seen.append((r.grant, toks[-1]))
         run(s, batch, toks)
         s.cache.check()
         if s.is_finished():
@@ -156,8 +156,25 @@ def test_running_request_without_a_page_sits_out_while_others_go_on():
     batch = s.schedule()
     assert batch == [b] and s.num_preemptions == 0   # a needs a new page and waits; b still has room
     run(s, batch, [3])
-    assert b.status == RequestStatus.FINISHED
+    assert b.phase == Phase.DONE
     assert s.schedule() == [a]
+
+
+def test_portions_of_a_multiple_where_a_part_asks_for_it():
+    """A mixer that works on blocks of 8 tokens: every portion but a request's last is a
+    multiple of 8, whatever the token limit and the free pages would allow."""
+    s = scheduler(num_pages=64, page_size=4, budget=21)
+    s.portion_multiple = 8
+    a, b = Request(list(range(30)), max_tokens=1), Request(list(range(9)), max_tokens=1)
+    s.add(a), s.add(b)
+    seen = []
+    while not s.is_finished():
+        batch = s.schedule()
+        seen.append([(r.request_id - a.request_id, r.grant) for r in batch])
+        run(s, batch, [5 if s.cache.length(r.request_id) + r.grant >= len(r.token_ids) else None for r in batch])
+    # 21 tokens a step: 16 of a (not 21); b's 9 do not fit whole into the 5 (then 7) tokens left,
+    # and a part of them would be no multiple of 8, so b waits; a's last 14 end it and need no rounding
+    assert seen == [[(0, 16)], [(0, 14)], [(1, 9)]]
 
 
 def test_nothing_running_and_no_page_is_an_error():
@@ -196,7 +213,7 @@ def test_finish_reasons(ignore_eos, min_tokens, tokens, reason, n_out):
                   sampling=SamplingParams(min_tokens=min_tokens))
     s.add(req)
     for tok in tokens:
-        if req.status == RequestStatus.FINISHED:
+        if req.phase == Phase.DONE:
             break
         run(s, s.schedule(), [tok])
     assert req.finish_reason == reason and req.num_output_tokens == n_out
@@ -209,9 +226,9 @@ def test_request_validation_and_forced_tokens():
     with pytest.raises(ValueError):
         Request([1], 0)
     r = Request([1, 2], 4, forced_tokens=[5, 6])
-    assert r.next_forced_token() == 5
+    assert r.forced_next() == 5
     r.token_ids += [5, 6]
-    assert r.next_forced_token() is None
+    assert r.forced_next() is None
     assert Request([1], 1, sampling=SamplingParams(seed=3)).seed == 3
 
 

@@ -104,8 +104,9 @@ def peak_tokens(steps, unit=64):
     return peak
 
 
-def replay(loaded, steps, check_cache=True):
-    """Run the steps through ``loaded.runner``; returns {(request, position): logits row}."""
+def replay(loaded, steps, check_cache=True, page_users=None):
+    """Run the steps through ``loaded.runner``; returns {(request, position): logits row}.
+    ``page_users`` (a dict) receives, per page of the first cache group, the requests that held it."""
     from qwen3_runtime_amd.engine.batch import StepEntry
 
     runner, cache = loaded.runner, loaded.cache
@@ -129,6 +130,10 @@ def replay(loaded, steps, check_cache=True):
             assert row == logits.shape[0]
         for e in s["entries"]:
             pos[e["id"]] += len(e["tokens"])
+            if page_users is not None and cache.groups:
+                for page in cache.block_table(0, e["id"]):
+                    if page >= 0:
+                        page_users.setdefault(page, set()).add(e["id"])
         for rid in s["end"]:
             cache.release(rid)
         if check_cache:
@@ -152,6 +157,30 @@ def plain_logits(folder, requests):
 def make_requests(vocab, lengths, seed=0):
     g = torch.Generator().manual_seed(seed)
     return {f"r{i}": torch.randint(0, vocab, (n,), generator=g).tolist() for i, n in enumerate(lengths)}
+
+
+def compare_rounding_noise(got, want, rms_bound=0.015, worst_bound=0.08):
+    """bfloat16 against the float64 plain implementation, in units of the logits' own spread.
+    Activations are rounded to 8 bits of mantissa some seven times per layer, which leaves an
+    error that behaves like noise: its root mean square is about 1 % of the logits' standard
+    deviation and its largest value over some 10^5 logits five times that. A fault in a page, a
+    mask or a portion's edge moves the logits of the positions it touches by a sizeable part of
+    their standard deviation, so the worst error is bounded at 8 % of it and the rms at 1.5 %."""
+    keys = sorted(want)
+    assert set(got) == set(want), f"{len(set(want) - set(got))} positions are missing"
+    w = torch.stack([want[k].double() for k in keys])
+    err = torch.stack([got[k].double() for k in keys]) - w
+    std = float(w.std())
+    rms = float(err.pow(2).mean().sqrt())
+    per_pos = err.abs().amax(dim=1)
+    worst = float(per_pos.max())
+    where = keys[int(per_pos.argmax())]
+    over = [keys[i] for i in torch.nonzero(per_pos >= worst_bound * std).flatten().tolist()]
+    assert worst < worst_bound * std, (
+        f"largest error {worst:.4f} at (request, position) {where}; logit deviation {std:.3f}; "
+        f"first position over the bound: {over[0]}")
+    assert rms < rms_bound * std, f"rms error {rms:.4f} against a logit deviation of {std:.3f}"
+    return rms / std, worst / std
 
 
 def compare(got, want, atol, rtol):
