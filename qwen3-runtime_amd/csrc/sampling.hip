@@ -8,7 +8,9 @@
 // and top_p are found by bisection on the value that bounds the kept set, not
 // by sorting; ids that tie with the bound are all kept.
 #include "common.h"
+#include "sampling.h"
 #include <math.h>
+#include <mutex>
 
 #define SAMPLE_THREADS 1024
 
@@ -81,26 +83,6 @@ extern "C" int qrt_argmax(const float* logits, int* out, int rows, int vocab, hi
   QRT_LAUNCH_CHECK("argmax");
   return 0;
 }
-
-// Per-request options live in the request's state slot, written once when the
-// request is admitted: fparams[slot] = {temperature, top_p, min_p, repetition,
-// presence, frequency, -, -}; iparams[slot] = {top_k, -}; seeds[slot] = {seed,
-// index of the next draw}. The kernel advances the draw index itself.
-struct SampleArgs {
-  const float* logits;      // [R, V]
-  float* work;              // [R, V] processed logits (scratch, returned to the caller)
-  const int* counts;        // [slots, V] occurrences of each id in prompt + output, or null
-  const int* slot;          // [R] state slot of each row
-  const float* fparams;     // [slots, 8]
-  const int* iparams;       // [slots, 2]
-  unsigned long long* seeds;  // [slots, 2]
-  int* out_token;           // [R]
-  float* out_logprob;       // [R]
-  int rows, vocab;
-  int write_work;           // also keep the processed logits of greedy rows
-  float* partials;          // [R, parts, 4]: maximum, sum of exp(value - maximum), first index of the maximum
-  int parts;                // > 0: the first pass ran in sample_first_pass_kernel, `parts` blocks per row
-};
 
 // The first pass over ids [lo, hi) of a row: penalties (reference:
 // qwen3_runtime/sampling.py:63-71) and temperature give the processed value (written to the
@@ -365,11 +347,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(SampleArgs a) {
   }
 }
 
-extern "C" int qrt_sample(const SampleArgs* args, hipStream_t stream) {
-  SampleArgs a = *args;
-  QRT_CHECK(a.rows >= 0 && a.vocab > 0, "sample: bad sizes");
-  if (a.rows == 0) return 0;
-  QRT_CHECK(a.parts >= 0 && a.parts <= 64 && (a.parts == 0 || a.partials), "sample: bad number of parts %d", a.parts);
+// both entry points: `a.partials` is already where the first pass may write
+static int launch_sample(const SampleArgs& a, hipStream_t stream) {
   if (a.parts > 0) {
     QRT_CHECK(a.rows <= 65535, "sample: %d rows in parts", a.rows);
     sample_first_pass_kernel<<<dim3(a.rows, a.parts), dim3(256), 0, stream>>>(a);
@@ -378,6 +357,73 @@ extern "C" int qrt_sample(const SampleArgs* args, hipStream_t stream) {
   sample_kernel<<<dim3(a.rows), dim3(SAMPLE_THREADS), 0, stream>>>(a);
   QRT_LAUNCH_CHECK("sample");
   return 0;
+}
+
+extern "C" int qrt_sample(const SampleArgs* args, hipStream_t stream) {
+  SampleArgs a = *args;
+  QRT_CHECK(a.rows >= 0 && a.vocab > 0, "sample: bad sizes");
+  if (a.rows == 0) return 0;
+  QRT_CHECK(a.parts >= 0 && a.parts <= 64 && (a.parts == 0 || a.partials), "sample: bad number of parts %d", a.parts);
+  return launch_sample(a, stream);
+}
+
+// ---- the entry point that allocates nothing (declared and described in sampling.h) ----------
+//
+// The partial results of the first pass live in this array, one copy per GPU, each at its own
+// address. In host code the array's name is only a handle for hipGetSymbolAddress, never an
+// address: kernels get the pointer that call returned for the current device.
+// No device code names the array (kernels get its address as an argument); it stays in the device
+// image, as a global symbol the runtime can look up, because host code below names it. (Marked
+// `used` it would stay a local symbol instead, which hipGetSymbolAddress cannot find.)
+static __device__ __align__(256) unsigned char scratch[QRT_SAMPLE_SCRATCH_BYTES];
+
+#define QRT_MAX_DEVICES 64
+static void* g_scratch_of_device[QRT_MAX_DEVICES] = {};
+static std::mutex g_scratch_mutex;
+
+// The current device's copy of `scratch`; looked up once per device, with that device current.
+static int scratch_for_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return qrt_fail("sample_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  QRT_CHECK(dev >= 0 && dev < QRT_MAX_DEVICES, "sample_noalloc: device %d is beyond the %d this library counts",
+            dev, QRT_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_of_device[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return qrt_fail("sample_noalloc: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_of_device[dev] = ptr;
+  }
+  *out = g_scratch_of_device[dev];
+  return 0;
+}
+
+// Optional: look the buffer up now (for the current device), so that the first sampling call,
+// which may sit inside a stream capture, finds it ready.
+extern "C" int qrt_sample_noalloc_setup() {
+  void* ptr = nullptr;
+  return scratch_for_current_device(&ptr);
+}
+
+extern "C" int qrt_sample_noalloc(const SampleArgs* args, hipStream_t stream) {
+  SampleArgs a = *args;
+  QRT_CHECK(a.rows >= 0 && a.vocab > 0, "sample_noalloc: bad sizes");
+  if (a.rows == 0) return 0;
+  QRT_CHECK(a.parts >= 0 && a.parts <= 64, "sample_noalloc: bad number of parts %d", a.parts);
+  const size_t need = (size_t)a.rows * (size_t)a.parts * 4 * sizeof(float);
+  QRT_CHECK(need <= QRT_SAMPLE_SCRATCH_BYTES,
+            "sample_noalloc: %d rows in %d parts need %zu bytes for the first pass's results; the buffer built "
+            "into the library holds %d (fewer parts, or qrt_sample with a buffer of the caller's)",
+            a.rows, a.parts, need, QRT_SAMPLE_SCRATCH_BYTES);
+  a.partials = nullptr;
+  if (a.parts > 0) {
+    void* ptr = nullptr;
+    if (scratch_for_current_device(&ptr) != 0) return -1;
+    a.partials = (float*)ptr;  // every entry [row, part] is written by the first pass before it is read
+  }
+  return launch_sample(a, stream);
 }
 
 // counts[slot[i], token[i]] += 1   (ids a request has seen: prompt and output)

@@ -111,7 +111,7 @@ def library_spec(name: str) -> tuple[list, list[str]]:
 def _digest(sources: list, defines: list[str]) -> str:
     h = hashlib.sha256()
     h.update(" ".join(FLAGS + defines).encode())
-    for name in list(sources) + ["common.h"]:
+    for name in list(sources) + sorted(p.name for p in CSRC.glob("*.h")):
         h.update(Path(name).name.encode())
         h.update((CSRC / name).read_bytes())  # an absolute path stays itself under "/"
     return h.hexdigest()
