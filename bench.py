@@ -7,18 +7,28 @@ A step is one decode step of the whole engine (schedule, graph replay or
 launches, sampling, copy of the sampled ids). The default run has the layer
 sizes of the Qwen3-4B configuration with seeded random weights, bfloat16, a
 batch of 8 requests whose prompts are 2,048 uniform-random ids, context limit
-8,192, pages of 16 tokens. W untimed steps, then exactly K timed steps between
-device synchronisations. Prints one JSON line: ``value`` is decoded tokens per
-second at batch 8; ``points`` adds batch 1 and 64; ``prefill`` is one
-2,048-token prompt in one step; ``roofline`` is the decode step's bytes (every
-weight once plus the cache of the live requests) over its time, against the
-published HBM peak.
+8,192, pages of 16 tokens. W untimed steps, then windows of exactly K timed
+steps between device synchronisations: three windows, the median one is
+reported and the spread of the three beside it (the reference's method: one
+warm-up and three trials, median and spread, bench/run_bench.py:164-182,
+bench/metrics.py:10-30). Prints one JSON line: ``value`` is decoded tokens per
+second at batch 8; ``points`` adds batch 1 and 64 (``point_rooflines`` their
+step times and fractions); ``prefill`` is one 2,048-token prompt in one step;
+``roofline`` is the decode step's bytes (every weight once plus the cache of
+the live requests) over its time, against the published HBM peak, with the
+bandwidth and the MFMA rate this device delivered in a microbenchmark beside
+the published figures (``measured_peak``).
+
+Other workloads: ``--workload mix`` (continuous batching of ``--requests``
+requests with prompts of 128 to 4,096 tokens, portions of 2,048, 256 outputs
+each) and any closed batch by ``--preset/--batch/--prompt-len/--context``.
 """
 
 from __future__ import annotations
 
 import argparse
 import json
+import statistics
 import sys
 import time
 
@@ -26,12 +36,63 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 # the reference's own steady decode rate at batch 8 (RTX 4090, 256-token prompts), for orientation
 REFERENCE_4090_B8_TOK_S = 740.0
+TRIALS = 3
+
+
+def say(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def spread(values) -> float:
+    """(max - min) / median, as the reference flags unstable trials (bench/metrics.py:10-30)."""
+    med = statistics.median(values)
+    return round((max(values) - min(values)) / med, 4) if med > 0 else 0.0
+
+
+def measure_device_peaks(device) -> dict:
+    """What this device delivers: GB/s reading 4 GiB once (far beyond every cache), and TFLOP/s
+    of bfloat16 32x32x16 MFMA instructions on registers with every SIMD busy. Best of five each."""
+    import ctypes
+
+    import torch
+
+    from qwen3_runtime_amd.ops import hip
+
+    lib = hip.load_library("peaks")
+    stream = hip.current_stream
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    nbytes = 4 << 30
+    buf = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+
+    def timed(launch) -> float:
+        best = float("inf")
+        for i in range(7):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            code = launch()
+            b.record()
+            b.synchronize()
+            if code != 0:
+                raise RuntimeError(lib.qrt_last_error().decode())
+            if i >= 2:
+                best = min(best, a.elapsed_time(b) * 1e-3)
+        return best
+
+    t_read = timed(lambda: lib.qrt_peak_read(ctypes.c_void_p(buf.data_ptr()), ctypes.c_size_t(nbytes),
+                                             ctypes.c_void_p(sink.data_ptr()), ctypes.c_int(256 * 64), stream()))
+    del buf
+    blocks, iters = 256 * 2, 20000
+    t_mfma = timed(lambda: lib.qrt_peak_mfma_bf16(ctypes.c_void_p(sink.data_ptr()), ctypes.c_int(blocks),
+                                                  ctypes.c_int(iters), stream()))
+    torch.cuda.empty_cache()
+    return {"hbm_gbs": round(nbytes / t_read / 1e9, 1),
+            "mfma_bf16_tflops": round(blocks * 4 * iters * 4 * 32768 / t_mfma / 1e12, 1)}
 
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--preset", default="qwen3_4b")
     ap.add_argument("--batch", type=int, default=8)
@@ -41,6 +102,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill measurement")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the microbenchmark of the device's own peaks")
+    ap.add_argument("--trials", type=int, default=TRIALS, help="timed windows of --steps steps each")
     ap.add_argument("--workload", default="decode", choices=["decode", "mix"],
                     help="decode: the closed batch (default). mix: --requests requests with prompts of 128 to 4,096 "
                          "tokens and 256 output tokens each through the scheduler, prompts read in portions of 2,048")
@@ -63,17 +126,26 @@ def main() -> int:
 
     cfg_full = preset(args.preset)
     cfg = cfg_full if args.layers is None else dataclasses.replace(cfg_full, num_hidden_layers=args.layers)
-    steps, warmup = args.steps, args.warmup
+    steps, warmup, trials = args.steps, args.warmup, max(1, args.trials)
     page = 16
     max_batch = args.batch if (args.no_points or args.prefill_only) else max(args.batch, 64)
     mix = args.workload == "mix"
     if mix:
         max_batch = args.requests
     budget = 2048  # tokens per step
+    dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    dev_name = "cuda:0"
+
+    peaks = None
+    if not args.no_peaks and not args.prefill_only:
+        peaks = measure_device_peaks(dev_name)
+        say(f"this device: {peaks['hbm_gbs']:.0f} GB/s read, {peaks['mfma_bf16_tflops']:.0f} TFLOP/s bf16 MFMA "
+            f"(published: {HBM_PEAK_GBS:.0f} GB/s, {MFMA_PEAK['bf16'] / 1e12:.0f} TFLOP/s)")
+
     # a request decodes while later ones are still read in: up to this many steps before the timed ones
     lead = lambda batch: batch * -(-args.prompt_len // budget)
-    per_req_tokens = args.prompt_len + steps + warmup + lead(max_batch) + 10
-    pages = max_batch * (-(-per_req_tokens // page) + 1)
+    per_req_tokens = args.prompt_len + trials * steps + warmup + lead(max_batch) + 10
+    pages = max_batch * (-(-min(per_req_tokens, args.context) // page) + 1)
     if mix:
         pages = max_batch * (-(-(4096 + 256) // page) + 1)
     t0 = time.time()
@@ -82,40 +154,69 @@ def main() -> int:
         max_num_seqs=max_batch, max_num_batched_tokens=budget, max_model_len=args.context,
         cuda_graph=not args.no_graph,
     )
-    print(f"[bench] model on device in {time.time() - t0:.1f} s, {engine.loaded.weight_bytes / 1e9:.2f} GB of weights",
-          file=sys.stderr, flush=True)
+    say(f"model on device in {time.time() - t0:.1f} s, {engine.loaded.weight_bytes / 1e9:.2f} GB of weights, "
+        f"{pages} pages")
     dev = engine.runner.device
     gen = torch.Generator().manual_seed(20260825)
     bytes_el = 2 if args.dtype == "bfloat16" else 4
+    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.kv_width * bytes_el
+    # every weight a step uses, once: a tied table is read once, as the head; an untied
+    # embedding table is only looked up
+    head_bytes = cfg.vocab_size * cfg.hidden_size * bytes_el
+    step_weight_bytes = engine.loaded.weight_bytes - (0 if cfg.tie_word_embeddings else head_bytes)
+    linear_flop_per_token = 2 * cfg.num_hidden_layers * (
+        cfg.hidden_size * (cfg.q_width + 2 * cfg.kv_width) + cfg.q_width * cfg.hidden_size
+        + 3 * cfg.hidden_size * cfg.intermediate_size)
 
-    def decode_run(batch: int, k: int, w: int):
-        """Prefill ``batch`` prompts, then time ``k`` decode steps after ``w`` warm-up steps."""
+    def roofline(step_seconds: float, kv_tokens: float) -> dict:
+        achieved = (step_weight_bytes + kv_tokens * kv_bytes_per_token) / step_seconds / 1e9
+        out = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+               "frac": round(achieved / HBM_PEAK_GBS, 4)}
+        if peaks:
+            out["measured_peak"] = peaks["hbm_gbs"]
+            out["frac_of_measured"] = round(achieved / peaks["hbm_gbs"], 4)
+        return out
+
+    def decode_run(batch: int, k: int, w: int, n_trials: int):
+        """Read ``batch`` prompts in, then ``n_trials`` windows of ``k`` timed decode steps after ``w``
+        warm-up steps. Returns the windows as (seconds, mean tokens in the cache), and the time the
+        prompts took."""
         prompts = torch.randint(0, cfg.vocab_size, (batch, args.prompt_len), generator=gen).tolist()
-        reqs = [engine.request(engine.add_request(p, max_tokens=k + w + lead(batch) + 8, sampling=SamplingParams()))
-                for p in prompts]
+        reqs = [engine.request(engine.add_request(p, max_tokens=n_trials * k + w + lead(batch) + 8,
+                                                  sampling=SamplingParams())) for p in prompts]
+        torch.cuda.synchronize(dev)
+        t = time.perf_counter()
         while any(len(r.token_ids) == r.prompt_len for r in reqs):
             engine.step()  # prompt portions until every request has its first token
+        torch.cuda.synchronize(dev)
+        fill = time.perf_counter() - t
         for _ in range(w):
             engine.step()
-        torch.cuda.synchronize(dev)
-        kv_tokens = sum(engine.cache.length(r.request_id) for r in reqs)
-        t = time.perf_counter()
-        for _ in range(k):
-            out = engine.step()
-            assert len(out) == batch and all(tok is not None for _, tok, _ in out)
-        torch.cuda.synchronize(dev)
-        dt = time.perf_counter() - t
-        kv_tokens = (kv_tokens + sum(engine.cache.length(r.request_id) for r in reqs)) / 2
+        windows = []
+        for _ in range(n_trials):
+            torch.cuda.synchronize(dev)
+            kv_before = sum(engine.cache.length(r.request_id) for r in reqs)
+            t = time.perf_counter()
+            for _ in range(k):
+                out = engine.step()
+                assert len(out) == batch and all(tok is not None for _, tok, _ in out)
+            torch.cuda.synchronize(dev)
+            dt = time.perf_counter() - t
+            kv_after = sum(engine.cache.length(r.request_id) for r in reqs)
+            windows.append((dt, (kv_before + kv_after) / 2))
         for r in reqs:
             engine.finish_request(r.request_id)
-        return dt, kv_tokens
+        return windows, fill
+
+    def median_window(windows):
+        return sorted(windows)[len(windows) // 2]
 
     def prefill_run():
         """One 2,048-token prompt through the step function, logits at its last token."""
         tokens = 2048
         ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=gen).tolist()
         times = []
-        for i in range(4):
+        for i in range(1 + trials):
             rid = f"prefill{i}"
             engine.cache.admit(rid)
             torch.cuda.synchronize(dev)
@@ -124,15 +225,18 @@ def main() -> int:
             torch.cuda.synchronize(dev)
             times.append(time.perf_counter() - t)
             engine.cache.release(rid)
-        pt = min(times[1:])
-        lin = 2 * tokens * cfg.num_hidden_layers * (
-            cfg.hidden_size * (cfg.q_width + 2 * cfg.kv_width) + cfg.q_width * cfg.hidden_size
-            + 3 * cfg.hidden_size * cfg.intermediate_size)
+        timed = times[1:]  # the first is the warm-up
+        pt = statistics.median(timed)
         attn = 2 * cfg.q_width * tokens * tokens * cfg.num_hidden_layers
         head = 2 * cfg.vocab_size * cfg.hidden_size
-        peak = MFMA_PEAK["bf16" if args.dtype == "bfloat16" else "fp32"]
-        return {"value": round(tokens / pt, 1), "tokens": tokens, "ms": round(pt * 1e3, 3),
-                "frac": round((lin + attn + head) / pt / peak, 4)}
+        flop = linear_flop_per_token * tokens + attn + head
+        peak = MFMA_PEAK[dtype_key]
+        out = {"value": round(tokens / pt, 1), "tokens": tokens, "ms": round(pt * 1e3, 3),
+               "frac": round(flop / pt / peak, 4), "trials": len(timed), "spread": spread(timed)}
+        if peaks and dtype_key == "bf16":
+            out["measured_peak_tflops"] = peaks["mfma_bf16_tflops"]
+            out["frac_of_measured"] = round(flop / pt / (peaks["mfma_bf16_tflops"] * 1e12), 4)
+        return out
 
     if args.prefill_only:
         print(json.dumps({"metric": "prefill tok/s, one 2,048-token prompt", "prefill": prefill_run()}), flush=True)
@@ -148,10 +252,16 @@ def main() -> int:
         t = time.perf_counter()
         reqs = [engine.request(engine.add_request(p, max_tokens=256, sampling=SamplingParams())) for p in prompts]
         n_steps = 0
+        floor_s = 0.0  # what the steps that ran would take at the published peaks
         stamps: dict[int, list[float]] = {r.request_id: [] for r in reqs}  # arrival time of every token
         while not engine.is_finished():
             out = engine.step()
             now = time.perf_counter() - t
+            stats = engine.last_step_stats
+            step_tokens = stats["prefill_tokens"] + stats["decode_tokens"]
+            kv_read = sum(engine.cache.length(rid) for rid in stats["req_ids"] if engine.cache.has(rid))
+            floor_s += max((step_weight_bytes + kv_read * kv_bytes_per_token) / (HBM_PEAK_GBS * 1e9),
+                           linear_flop_per_token * step_tokens / MFMA_PEAK[dtype_key])
             for rid, tok, _done in out:
                 if tok is not None:
                     stamps[rid].append(now)
@@ -174,29 +284,32 @@ def main() -> int:
             "ttft_ms": {"p50": pick(ttft, 0.5), "p99": pick(ttft, 0.99)},
             "tpot_ms": {"p50": pick(tpot, 0.5), "p99": pick(tpot, 0.99)},
             "itl_ms": {"p50": pick(itl, 0.5), "p99": pick(itl, 0.99)},
-            "preemptions": engine.scheduler.num_preemptions, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            # each step priced at max(bytes / HBM peak, flop / MFMA peak), summed, over the time taken
+            "roofline": {"bound": "per step: hbm or mfma", "floor_s": round(floor_s, 3), "frac": round(floor_s / dt, 4)},
+            "measured_peak": peaks,
+            "preemptions": engine.scheduler.num_preemptions, "dtype": dtype_key,
             "data": "synthetic: uniform-random token ids and lengths, seeded random weights",
             "config": {"model": f"{args.preset} shape", "layers": cfg.num_hidden_layers, "max_num_seqs": max_batch,
                        "max_num_batched_tokens": budget, "page_size": page, "hip_graph": not args.no_graph},
         }), flush=True)
         return 0
 
-    dt, kv_tokens = decode_run(args.batch, steps, warmup)
+    windows, fill_s = decode_run(args.batch, steps, warmup, trials)
+    dt, kv_tokens = median_window(windows)
     ms_per_step = dt / steps * 1e3
     value = args.batch * steps / dt
-    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.kv_width * bytes_el
-    # every weight the step uses, once: the tied table is read once, as the head
-    head_bytes = cfg.vocab_size * cfg.hidden_size * bytes_el
-    step_weight_bytes = engine.loaded.weight_bytes if cfg.tie_word_embeddings else engine.loaded.weight_bytes - head_bytes
-    step_bytes = step_weight_bytes + kv_tokens * kv_bytes_per_token
-    achieved = step_bytes / (dt / steps) / 1e9
 
-    points, prefill = {}, None
+    points, point_rooflines, prefill = {}, {}, None
     if not args.no_points:
         for b in (1, 64):
             k = min(steps, 64)
-            d, _ = decode_run(b, k, min(warmup, 8))
+            w, _ = decode_run(b, k, min(warmup, 8), trials)
+            d, kv = median_window(w)
             points[f"decode_b{b}"] = round(b * k / d, 1)
+            r = roofline(d / k, kv)
+            point_rooflines[f"decode_b{b}"] = {"ms_per_step": round(d / k * 1e3, 4), "frac": r["frac"],
+                                               "achieved_gbs": r["achieved"],
+                                               "spread": spread([x[0] for x in w])}
         prefill = prefill_run()
 
     shape_name = {"qwen3_4b": "Qwen3-4B", "qwen3_8b": "Qwen3-8B", "qwen3_32b": "Qwen3-32B"}.get(args.preset, args.preset)
@@ -211,7 +324,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "dtype": dtype_key,
         "data": "synthetic: uniform-random token ids, seeded random weights N(0, 0.02), norms 1.0",
         "config": {
             "model": f"{args.preset} shape",
@@ -231,14 +344,24 @@ def main() -> int:
             "hip_graph": not args.no_graph,
             "parallelism": "single GPU",
         },
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "trials": {"windows": trials, "steps_each": steps, "reported": "median window",
+                   "ms_per_step": [round(w[0] / steps * 1e3, 4) for w in windows],
+                   "spread": spread([w[0] for w in windows])},
+        "roofline": roofline(dt / steps, kv_tokens),
+        # reading the prompts in, portions of 2,048 tokens beside the decoding of those already in
+        "prompt_phase": {"tokens": args.batch * args.prompt_len, "seconds": round(fill_s, 3),
+                         "tok_s": round(args.batch * args.prompt_len / fill_s, 1)},
+        "env": {"gpu": torch.cuda.get_device_name(dev), "torch": torch.__version__, "hip": torch.version.hip,
+                "hbm_gib": round(torch.cuda.get_device_properties(dev).total_memory / 2**30, 1)},
     }
+    if peaks:
+        line["measured_peak"] = peaks
     if args.preset == "qwen3_4b" and args.batch == 8 and args.prompt_len == 2048:
         line["vs_reference_rtx4090_batch8"] = round(value / REFERENCE_4090_B8_TOK_S, 2)
     if prefill is not None:
         line["prefill"] = prefill
         line["points"] = points
+        line["point_rooflines"] = point_rooflines
     print(json.dumps(line), flush=True)
     return 0
 

@@ -47,7 +47,7 @@ def register_library(name: str, sources, defines=()) -> None:
     include ``common.h`` of this package, which is on the include path, and then link
     ``runtime.hip`` for ``qrt_fail`` / ``qrt_last_error`` by listing it as ``"runtime.hip"``).
     Registering the same name with the same sources again is allowed."""
-    if name == "core" or name.startswith("attn_bf16_d"):
+    if name in ("core", "peaks") or name.startswith("attn_bf16_d"):
         raise BuildError(f"{name!r} is a library of the engine's own")
     paths = [CSRC / s if not Path(s).is_absolute() else Path(s) for s in sources]
     for path in paths:
@@ -98,6 +98,8 @@ def library_spec(name: str) -> tuple[list, list[str]]:
     """Sources (names under ``csrc``, or paths) and extra defines of a library name."""
     if name == "core":
         return CORE_SOURCES, []
+    if name == "peaks":  # the device's own bandwidth and MFMA rate, for the measurements
+        return ["runtime.hip", "peaks.hip"], []
     if name in _REGISTERED:
         return list(_REGISTERED[name][0]), list(_REGISTERED[name][1])
     if name.startswith("attn_bf16_d"):
@@ -174,5 +176,5 @@ def build_library(name: str, force: bool = False) -> Path:
 
 def build_all(head_dims=(16, 32, 48, 64, 80, 96, 112, 128, 256), force: bool = True) -> list[Path]:
     """Every library the tests, the smoke run and the measurements load."""
-    names = ["core"] + [f"attn_bf16_d{d}" for d in head_dims] + registered_libraries()
+    names = ["core", "peaks"] + [f"attn_bf16_d{d}" for d in head_dims] + registered_libraries()
     return [build_library(n, force=force) for n in names]

@@ -36,11 +36,38 @@ def test_bench_line_has_the_contract_fields():
     assert rec["n_gpus"] == 1 and rec["steps"] == 8 and rec["warmup"] == 2 and rec["higher_is_better"] is True
     assert len(rec["config"]) <= 20 and all(not isinstance(v, (dict, list)) for v in rec["config"].values())
     assert rec["config"]["layers"] == 2 and rec["config"]["layers_of_full_model"] == 36
-    assert set(rec["prefill"]) == {"value", "tokens", "ms", "frac"} and rec["prefill"]["tokens"] == 2048
+    assert {"value", "tokens", "ms", "frac"} <= set(rec["prefill"]) and rec["prefill"]["tokens"] == 2048
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0
     assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / rec["roofline"]["peak"]) < 1e-3
     assert set(rec["points"]) == {"decode_b1", "decode_b64"}
+    assert all(isinstance(v, float) for v in rec["points"].values())
     assert abs(rec["value"] - 8 * 1000.0 / rec["ms_per_step"]) / rec["value"] < 0.01
+
+    # the arithmetic behind the fractions, recomputed here from the sizes the line names
+    c = rec["config"]
+    h, d, i, v, layers = c["hidden"], c["head_dim"], c["intermediate"], c["vocab"], c["layers"]
+    q, kv = c["heads"] * d, c["kv_heads"] * d
+    per_layer = h * (q + 2 * kv) + q * h + 3 * h * i + 2 * h + 2 * d       # matrices, two norms, q/k norms
+    weight_bytes = 2 * (v * h + layers * per_layer + h)                    # tied table once, final norm
+    kv_per_token = 2 * layers * kv * 2
+    step_s = rec["ms_per_step"] * 1e-3
+    # each of the 8 requests holds its 2,048-token prompt and between 1 and ~100 decoded tokens
+    low = (weight_bytes + 8 * 2049 * kv_per_token) / step_s / 1e9
+    high = (weight_bytes + 8 * 2150 * kv_per_token) / step_s / 1e9
+    assert low * 0.999 <= rec["roofline"]["achieved"] <= high * 1.001, (low, rec["roofline"]["achieved"], high)
+    flop = 2048 * 2 * layers * (h * (q + 2 * kv) + q * h + 3 * h * i) + 2 * q * 2048 * 2048 * layers + 2 * v * h
+    assert abs(rec["prefill"]["frac"] - flop / (rec["prefill"]["ms"] * 1e-3) / 2.5e15) < 2e-4
+    assert abs(rec["prefill"]["value"] - 2048 / (rec["prefill"]["ms"] * 1e-3)) / rec["prefill"]["value"] < 1e-3
+    for b, point in rec["point_rooflines"].items():
+        batch = int(b.rsplit("b", 1)[1])
+        assert abs(rec["points"][b] - batch * 1000.0 / point["ms_per_step"]) / rec["points"][b] < 0.01
+        floor = (weight_bytes + batch * 2049 * kv_per_token) / (point["ms_per_step"] * 1e-3) / 1e9 / 8000.0
+        assert floor * 0.999 <= point["frac"] <= floor * 1.06
+    # the device's own peaks stand beside the published ones, and are plausible for this part
+    assert 2000 < rec["measured_peak"]["hbm_gbs"] < 8000 and 500 < rec["measured_peak"]["mfma_bf16_tflops"] < 2600
+    assert rec["roofline"]["measured_peak"] == rec["measured_peak"]["hbm_gbs"]
+    assert rec["trials"]["windows"] == 3 and len(rec["trials"]["ms_per_step"]) == 3
+    assert min(rec["trials"]["ms_per_step"]) <= rec["ms_per_step"] <= max(rec["trials"]["ms_per_step"])
 
 
 @pytest.mark.gpu
