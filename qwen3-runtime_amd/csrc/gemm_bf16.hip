@@ -156,7 +156,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t*
       const int s = s0 + u * NW;
       if (s < steps) {  // uniform over the wave
 #pragma unroll
-        for (int t = 0; t < WT; ++t) w[u][t] = *(const bf16x8_t*)(wrow[t] + (size_t)s * WSTEP);
+        for (int t = 0; t < WT; ++t) w[u][t] = load_once8(wrow[t] + (size_t)s * WSTEP);
 #pragma unroll
         for (int b = 0; b < MB; ++b) a[u][b] = avalid[b] ? *(const bf16x8_t*)(arow[b] + (s << 5)) : zero;
       }

@@ -31,6 +31,8 @@ FLAGS = [
     # packed float32 instructions stay off: some of their forms have returned wrong results
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# further hipcc flags (for instance -D switches of a kernel under tuning); part of the libraries' hash
+FLAGS += os.environ.get("QWEN3_RUNTIME_AMD_HIPCC_FLAGS", "").split()
 CORE_SOURCES = ["runtime.hip", "elementwise.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_f32.hip", "sampling.hip"]
 
 

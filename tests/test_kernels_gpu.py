@@ -226,6 +226,31 @@ def test_product_for_the_residual_may_come_in_planes(m, n, k):
     close(yc, ya[rows.long()], 0, 0)
 
 
+@pytest.mark.parametrize("m", [1, 8, 64])
+def test_vocabulary_head_at_its_real_size(m):
+    """The head of the 4B and 8B models, 151,936 x 2,560, through the dispatch a decode step uses
+    (tile-major copy; the few-row kernel with two row tiles per block up to 16 rows, the kernel
+    that shares activations with eight tiles per block for 64), float32 out, against a float64
+    product of the same bfloat16 values computed on the device."""
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    ops = HipOps()
+    n, k = 151936, 2560
+    x = rnd(m, k, dtype=torch.bfloat16, seed=5)
+    g = torch.Generator(device=DEV).manual_seed(17)
+    w = (0.02 * torch.randn(n, k, generator=g, device=DEV, dtype=torch.float32)).to(torch.bfloat16)
+    ops.prepare_weight(w)
+    assert ops._tiled_copy(w) is not None and ops._own_kernel(m, k, ops._tiled_copy(w), "whole") == (1 if m <= 16 else 2)
+    got = ops.linear(x, w, out_f32=True)
+    want = torch.empty((m, n), dtype=torch.float64, device=DEV)
+    for lo in range(0, n, 16384):                       # in pieces: the float64 copy of W is 3 GB otherwise
+        want[:, lo: lo + 16384] = x.double() @ w[lo: lo + 16384].double().T
+    err = (got.double() - want).abs()
+    # entries are sums of 2,560 products of size 0.02: about one in size; float32 sums err by 1e-5 or so
+    assert 0.5 < float(want.abs().mean()) < 1.5 and float(err.max()) < 2e-4, float(err.max())
+    assert torch.equal(got.argmax(-1), want.argmax(-1))
+
+
 def test_gemm_bf16_large_uses_blas_and_agrees(ops):
     x, w = rnd(300, 512, dtype=torch.bfloat16, seed=1), rnd(640, 512, dtype=torch.bfloat16, seed=2, scale=0.05)
     close(ops.linear(x, w), x.double() @ w.double().T, 3e-2, 3e-2)

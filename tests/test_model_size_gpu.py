@@ -142,3 +142,27 @@ def test_model_sized_decode_graph_equals_eager(sized_folders):
         del llm
         torch.cuda.empty_cache()
     assert outs[0] == outs[1]
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_the_2048_token_prompt_the_measurement_times(sized_folders, dtype):
+    """One 2,048-token prompt in one step at the 4B layer sizes, the step whose time is reported as
+    prefill throughput: the vendor products at 2,048 rows, the prompt attention through LDS with
+    128 row tiles and their work list, the wide q/k kernel. Logits at every 16th position and at
+    the last ones against the plain implementation."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg, folder = sized_folders["qwen3_4b"]
+    reqs = traces.make_requests(cfg.vocab_size, [2048], seed=44)
+    want_all = traces.plain_logits(folder, reqs)
+    wanted = sorted(set(range(0, 2048, 16)) | set(range(2040, 2048)))
+    steps = [{"step": 0, "entries": [{"id": "r0", "tokens": reqs["r0"], "want": wanted}], "end": ["r0"]}]
+    engine_cfg = EngineConfig(page_size=16, num_pages=128, max_num_seqs=1, max_num_batched_tokens=2048, dtype=dtype,
+                              device="cuda:0", hip_graph=False)
+    got = traces.replay(load(folder, engine_cfg), steps)
+    want = {("r0", p): want_all[("r0", p)] for p in wanted}
+    if dtype == "float32":
+        traces.compare(got, want, **TOL_F32)
+    else:
+        check_rounding_noise(got, want)
