@@ -270,12 +270,72 @@ class HipOps:
             # many rows: the vendor library; both accumulate in float32
             if out_f32:
                 return torch.mm(x, w.t(), out_dtype=torch.float32)
-            return torch.matmul(x, w.t())
+            return self._library_product(x, w)
         out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
         self._check(self.lib, self.lib.qrt_gemm_bf16(
             _ptr(x), _ptr(tiled if kernel else w), _ptr(out), F32 if out_f32 else BF16,
             c_int(m), c_int(n), c_int(k), c_int(0), c_int(kernel), c_int(1), _stream()))
         return out
+
+    # rows from which a library product is tried in two column chunks
+    library_split_min_rows = 256
+
+    def _library_product(self, x, w):
+        """``x @ w.T`` by the vendor library, in one call or in two over column chunks of the result.
+
+        The library's kernels work on tiles of the result (256 x 256 for these shapes), and a
+        result whose tiles do not fill the 256 compute units a whole number of times leaves
+        them idle in the last round: 2,048 x 19,456 is 608 tiles, 2.4 rounds. A first chunk of
+        columns that fills whole rounds and a second call for the rest took 175 us instead of
+        210 there, and 293 instead of 393 at 4,096 rows. Whether it pays depends on the
+        library's own choices, so each shape (rows in units of 256, N, K) is timed both ways
+        the first time it is met, outside stream capture, and the faster way is kept."""
+        m, k = x.shape
+        n = w.shape[0]
+        split = self._library_split(x, w)
+        if not split:
+            return torch.matmul(x, w.t())
+        out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+        torch.mm(x, w[:split].t(), out=out[:, :split])
+        torch.mm(x, w[split:].t(), out=out[:, split:])
+        return out
+
+    def _library_split(self, x, w) -> int:
+        m, k = x.shape
+        n = w.shape[0]
+        if m < self.library_split_min_rows:
+            return 0
+        row_tiles = -(-m // 256)
+        per_round = 256 * max(1, 256 // row_tiles)  # columns whose tiles fill the compute units once
+        split = (n // per_round) * per_round
+        if not 0 < split < n:
+            return 0
+        plans = self.__dict__.setdefault("_library_plans", {})
+        key = (row_tiles, n, k)
+        if key not in plans:
+            if torch.cuda.is_current_stream_capturing():
+                return 0  # not timed yet, and no timing inside a capture
+            out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+
+            def whole():
+                torch.mm(x, w.t(), out=out)
+
+            def chunked():
+                torch.mm(x, w[:split].t(), out=out[:, :split])
+                torch.mm(x, w[split:].t(), out=out[:, split:])
+
+            def timed(fn):
+                fn()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for _ in range(3):
+                    fn()
+                b.record()
+                b.synchronize()
+                return a.elapsed_time(b)
+
+            plans[key] = split if timed(chunked) < 0.97 * timed(whole) else 0
+        return plans[key]
 
     def _own_kernel(self, m: int, k: int, tiled, form: str) -> int | None:
         """Which of the library's kernels multiplies ``m`` rows by this weight: 0 the few-row

@@ -257,6 +257,27 @@ def test_gemm_bf16_large_uses_blas_and_agrees(ops):
     close(ops.linear(x, w, out_f32=True), x.double() @ w.double().T, 1e-3, 1e-3)
 
 
+def test_library_product_in_two_column_chunks():
+    """Products with many rows go to the vendor library, whole or as two calls over column chunks
+    of one result tensor, whichever was faster when the shape was first met. Both ways, and the
+    way chosen, give the float64 product."""
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    ops = HipOps()
+    m, n, k = 300, 33000, 64                       # two row tiles: 32,768 columns fill the chip once
+    x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
+    want = x.double() @ w.double().T
+    close(ops.linear(x, w), want, 3e-2, 3e-2)      # timed both ways now, one of them kept
+    assert ops._library_plans[(2, n, k)] in (0, 32768)
+    for split in (0, 32768):
+        ops._library_plans[(2, n, k)] = split
+        got = ops.linear(x, w)
+        assert got.is_contiguous() and got.shape == (m, n)
+        close(got, want, 3e-2, 3e-2)
+    assert ops._library_split(x[:200], w) == 0     # few rows: never split
+    assert ops._library_split(x, w[:30000]) == 0   # fewer columns than one round
+
+
 def test_float32_weight_with_bfloat16_activations_stays_float32(ops):
     x, w = rnd(5, 64, dtype=torch.bfloat16), rnd(48, 64, scale=0.1)
     close(ops.linear(x, w, out_f32=True), x.double() @ w.double().T, 1e-5, 1e-5)
