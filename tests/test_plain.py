@@ -154,25 +154,139 @@ def test_whole_model_shift_of_positions_and_hand_computed_layer(model_folders):
     torch.testing.assert_close(got, want)
 
 
+def _library_attention_layer(x, wq, wk, pos, theta, eps):
+    """One head, identity projections, written with library routines only: F.rms_norm, a complex
+    multiplication for the rotation, F.scaled_dot_product_attention."""
+    d = x.shape[-1]
+
+    def rotate(v):
+        inv = 1.0 / theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d)
+        ang = (pos.float()[:, None] * inv[None, :]).double()
+        z = torch.complex(v[:, : d // 2], v[:, d // 2:]) * torch.polar(torch.ones_like(ang), ang)
+        return torch.cat((z.real, z.imag), -1)
+
+    q = rotate(F.rms_norm(x, (d,), wq, eps))
+    k = rotate(F.rms_norm(x, (d,), wk, eps))
+    return F.scaled_dot_product_attention(q[None, None], k[None, None], x[None, None], is_causal=True)[0, 0]
+
+
 def test_q_norm_comes_before_the_rotation():
-    """With a non-uniform norm weight, norm-then-rotate differs from rotate-then-norm."""
+    """With a non-uniform norm weight, norm-then-rotate differs from rotate-then-norm; the
+    expected values come from library routines, not from the plain functions."""
     torch.manual_seed(6)
     d = 8
     cfg = dict(num_attention_heads=1, num_key_value_heads=1, head_dim=d, hidden_size=d, rms_norm_eps=1e-6,
                rope_theta=10.0)
     eye = torch.eye(d).double()
     wq = torch.tensor([0.1, 0.9, 0.2, 0.8, 0.3, 0.7, 0.4, 0.6]).double()
+    wk = torch.tensor([1.0, 0.5, 1.5, 0.7, 0.9, 1.1, 0.6, 1.3]).double()
     w = {"a.q_proj.weight": eye, "a.k_proj.weight": eye, "a.v_proj.weight": eye, "a.o_proj.weight": eye,
-         "a.q_norm.weight": wq, "a.k_norm.weight": torch.ones(d).double()}
+         "a.q_norm.weight": wq, "a.k_norm.weight": wk}
     x = torch.randn(4, d).double()
     pos = torch.tensor([0, 3, 4, 9])
     got = P.attention_layer(x, w, "a", cfg, pos)
-    q = P.rope_neox(P.rms_norm(x.view(4, 1, d), wq, 1e-6), pos, 10.0)
-    k = P.rope_neox(P.rms_norm(x.view(4, 1, d), torch.ones(d).double(), 1e-6), pos, 10.0)
-    want = P.causal_attention(q, k, x.view(4, 1, d))
-    torch.testing.assert_close(got, want)
+    torch.testing.assert_close(got, _library_attention_layer(x, wq, wk, pos, 10.0, 1e-6))
+    # the plausible mistake: rotate first, then norm
     q_wrong = P.rms_norm(P.rope_neox(x.view(4, 1, d), pos, 10.0), wq, 1e-6)
-    assert (P.causal_attention(q_wrong, k, x.view(4, 1, d)) - got).abs().max() > 1e-3
+    k_right = P.rope_neox(P.rms_norm(x.view(4, 1, d), wk, 1e-6), pos, 10.0)
+    assert (P.causal_attention(q_wrong, k_right, x.view(4, 1, d)) - got).abs().max() > 1e-3
+
+
+def _tiny_model(layers=2, tied=False, seed=0):
+    """A hand-sized model with every norm weight different, in float64."""
+    g = torch.Generator().manual_seed(seed)
+    h, nq, nkv, d, i, v = 12, 2, 1, 4, 10, 17
+    cfg = dict(num_hidden_layers=layers, hidden_size=h, num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d,
+               intermediate_size=i, vocab_size=v, rms_norm_eps=1e-5, rope_theta=100.0, tie_word_embeddings=tied)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float64)
+    w = {"model.embed_tokens.weight": rnd(v, h), "model.norm.weight": 1 + 0.5 * rnd(h), "lm_head.weight": rnd(v, h)}
+    for l in range(layers):
+        p = f"model.layers.{l}"
+        w.update({f"{p}.input_layernorm.weight": 1 + 0.5 * rnd(h), f"{p}.post_attention_layernorm.weight": 1 + 0.5 * rnd(h),
+                  f"{p}.self_attn.q_proj.weight": rnd(nq * d, h), f"{p}.self_attn.k_proj.weight": rnd(nkv * d, h),
+                  f"{p}.self_attn.v_proj.weight": rnd(nkv * d, h), f"{p}.self_attn.o_proj.weight": rnd(h, nq * d),
+                  f"{p}.self_attn.q_norm.weight": 1 + 0.5 * rnd(d), f"{p}.self_attn.k_norm.weight": 1 + 0.5 * rnd(d),
+                  f"{p}.mlp.gate_proj.weight": rnd(i, h), f"{p}.mlp.up_proj.weight": rnd(i, h),
+                  f"{p}.mlp.down_proj.weight": rnd(h, i)})
+    return cfg, w
+
+
+def test_the_order_of_the_layers_parts_by_special_cases_that_reduce_to_library_routines():
+    """Where the norms stand, what the residual adds, the final norm and the head, each pinned by a
+    model in which all but one sub-layer is switched off (its output matrix zeroed), so that the
+    logits can be written with F.rms_norm, F.silu and F.linear alone. A post-norm block, a residual
+    taken from the normed tensor, the feed-forward behind the wrong norm, a missing final norm or
+    the embedding used where the model has a head of its own each fail one of these."""
+    eps = 1e-5
+    norm = lambda x, wt: F.rms_norm(x, (x.shape[-1],), wt, eps)
+    ids = torch.tensor([3, 11, 5, 3, 16])
+
+    # 1. every sub-layer off: logits = head(final_norm(embedding))
+    cfg, w = _tiny_model(layers=2)
+    for l in range(2):
+        w[f"model.layers.{l}.self_attn.o_proj.weight"].zero_()
+        w[f"model.layers.{l}.mlp.down_proj.weight"].zero_()
+    e = w["model.embed_tokens.weight"][ids]
+    torch.testing.assert_close(P.forward(cfg, w, ids), F.linear(norm(e, w["model.norm.weight"]), w["lm_head.weight"]))
+    cfg_tied = dict(cfg, tie_word_embeddings=True)
+    torch.testing.assert_close(P.forward(cfg_tied, w, ids),
+                               F.linear(norm(e, w["model.norm.weight"]), w["model.embed_tokens.weight"]))
+
+    # 2. only the feed-forward of layer 1 on: h = e + down(silu(gate n) * up n), n = post-attention norm of e
+    cfg, w = _tiny_model(layers=2, seed=1)
+    for l in range(2):
+        w[f"model.layers.{l}.self_attn.o_proj.weight"].zero_()
+    w["model.layers.0.mlp.down_proj.weight"].zero_()
+    e = w["model.embed_tokens.weight"][ids]
+    p = "model.layers.1"
+    n = norm(e, w[f"{p}.post_attention_layernorm.weight"])
+    ff = F.linear(F.silu(F.linear(n, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(n, w[f"{p}.mlp.up_proj.weight"]),
+                  w[f"{p}.mlp.down_proj.weight"])
+    want = F.linear(norm(e + ff, w["model.norm.weight"]), w["lm_head.weight"])
+    torch.testing.assert_close(P.forward(cfg, w, ids), want)
+    for wrong in (F.linear(norm(n + ff, w["model.norm.weight"]), w["lm_head.weight"]),           # residual from the normed tensor
+                  F.linear(norm(norm(e + ff, w[f"{p}.post_attention_layernorm.weight"]), w["model.norm.weight"]),
+                           w["lm_head.weight"])):                                                 # post-norm
+        assert (wrong - want).abs().max() > 1e-2
+
+    # 3. only the attention of layer 0 on, one token (attention then returns its value):
+    #    h = e + o(repeat(v(input norm of e)))
+    cfg, w = _tiny_model(layers=2, seed=2)
+    for l in range(2):
+        w[f"model.layers.{l}.mlp.down_proj.weight"].zero_()
+    w["model.layers.1.self_attn.o_proj.weight"].zero_()
+    one = ids[:1]
+    e = w["model.embed_tokens.weight"][one]
+    p = "model.layers.0"
+    n = norm(e, w[f"{p}.input_layernorm.weight"])
+    v = F.linear(n, w[f"{p}.self_attn.v_proj.weight"]).view(1, 1, 4).repeat_interleave(2, 1).reshape(1, 8)
+    want = F.linear(norm(e + F.linear(v, w[f"{p}.self_attn.o_proj.weight"]), w["model.norm.weight"]), w["lm_head.weight"])
+    torch.testing.assert_close(P.forward(cfg, w, one), want)
+
+    # 4. both sub-layers of one layer on, two tokens: the feed-forward sees the stream after the
+    #    attention's add, through the post-attention norm (attention from library routines)
+    cfg, w = _tiny_model(layers=1, seed=3)
+    two = ids[:2]
+    e = w["model.embed_tokens.weight"][two]
+    n = norm(e, w[f"{p}.input_layernorm.weight"])
+    d = 4
+    def heads(x, k):
+        return x.view(2, k, d)
+    def rotate(x):
+        inv = 1.0 / 100.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d)
+        ang = (torch.arange(2).float()[:, None] * inv[None, :]).double()[:, None, :]
+        z = torch.complex(x[..., : d // 2], x[..., d // 2:]) * torch.polar(torch.ones_like(ang), ang)
+        return torch.cat((z.real, z.imag), -1)
+    q = rotate(F.rms_norm(heads(F.linear(n, w[f"{p}.self_attn.q_proj.weight"]), 2), (d,), w[f"{p}.self_attn.q_norm.weight"], eps))
+    k = rotate(F.rms_norm(heads(F.linear(n, w[f"{p}.self_attn.k_proj.weight"]), 1), (d,), w[f"{p}.self_attn.k_norm.weight"], eps))
+    v = heads(F.linear(n, w[f"{p}.self_attn.v_proj.weight"]), 1)
+    attn = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.repeat_interleave(2, 1).transpose(0, 1)[None],
+                                          v.repeat_interleave(2, 1).transpose(0, 1)[None], is_causal=True)[0]
+    h1 = e + F.linear(attn.transpose(0, 1).reshape(2, 8), w[f"{p}.self_attn.o_proj.weight"])
+    n2 = norm(h1, w[f"{p}.post_attention_layernorm.weight"])
+    h2 = h1 + F.linear(F.silu(F.linear(n2, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(n2, w[f"{p}.mlp.up_proj.weight"]),
+                       w[f"{p}.mlp.down_proj.weight"])
+    torch.testing.assert_close(P.forward(cfg, w, two), F.linear(norm(h2, w["model.norm.weight"]), w["lm_head.weight"]))
 
 
 def test_engine_formulation_equals_plain_on_cpu(model_folders):
