@@ -268,7 +268,7 @@ __device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int b
 // operand traffic per MFMA by RT.
 template <int RT, bool P2>
 __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(AttnTileArgs a) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = uniform_wave_number();
   const int r16 = lane & 15, quad = lane >> 4;
   // blocks of one tile are neighbours in the launch order, one per key head: with as many key
   // heads as XCDs, a head's keys and values stay in one XCD's L2
@@ -408,7 +408,7 @@ constexpr int STAGE_ELEMS = 32 * KROW + D * VROW;
 template <int RT, bool P2>
 __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTileArgs a) {
   extern __shared__ bf16_t lds_kv[];  // [2][STAGE_ELEMS]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = uniform_wave_number();
   const int r16 = lane & 15, quad = lane >> 4;
   const int tile = blockIdx.x / a.nkv, kvh = blockIdx.x - tile * a.nkv, split = blockIdx.z;
   const int seq = a.tile_seq[tile];
@@ -486,7 +486,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   const size_t page_stride = (size_t)a.nkv * ps * D;  // elements per page, keys and values alike
   const bf16_t* k_head = a.k_cache + (size_t)kvh * ps * D;
   const bf16_t* v_head = a.v_cache + (size_t)kvh * D * ps;
-  const int w8 = 8 * __builtin_amdgcn_readfirstlane(wave);  // this wave's group within a block
+  const int w8 = 8 * wave;  // this wave's group within a block
   constexpr int LANE_PIECES = (D + 63) / 64;   // 16-byte pieces per lane, of keys and of values
   constexpr bool ALL_LANES = D % 64 == 0;
   struct Pieces { bf16x8_t k[LANE_PIECES], v[LANE_PIECES]; };
@@ -702,7 +702,7 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
   float* lds_l = lds + DW * 16;       // [DW][16]
   float* lds_o = lds + 2 * DW * 16;   // [DW][16][D]
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = uniform_wave_number();
   const int r16 = lane & 15, quad = lane >> 4;
   // every sequence is one tile here, so without a list the block's number is the sequence's: one
   // dependent load less before the first key arrives. A list names the sequences of a launch

@@ -34,6 +34,13 @@ int qrt_fail(const char* fmt, ...);
     if (e_ != hipSuccess) return qrt_fail("%s: launch failed: %s", name, hipGetErrorString(e_)); \
   } while (0)
 
+// The wave's number within its block, in a scalar register: what follows from it (the wave's rows,
+// its share of a loop) is then the same for the whole wave to the compiler too, and branches on it
+// become scalar branches. For kernels with MFMA instructions this is needed, not only faster:
+// MFMA does not look at the EXEC mask, so one inside a branch that the compiler lowered to an
+// EXEC mask of zeros, without a jump over it, runs all the same, on registers never loaded.
+__device__ __forceinline__ int uniform_wave_number() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
+
 // Eight bfloat16 of a matrix that a step reads exactly once (weights streamed past few rows of
 // activations): a non-temporal load, which leaves the caches to data that is read again. A plain
 // read of 4 GiB runs at 6.1 TB/s on this device, a non-temporal one at 6.9; the few-row products

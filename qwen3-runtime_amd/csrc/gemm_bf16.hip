@@ -29,7 +29,7 @@ __device__ __forceinline__ bf16x8_t load_k8(const bf16_t* __restrict__ row, int 
 template <int MT, int NT, bool ALIGNED, typename TO>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                                          TO* __restrict__ C, int M, int N, int K) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = uniform_wave_number();
   const int r16 = lane & 15, quad = lane >> 4;
   const int m0 = blockIdx.y * (16 * MT);
   const int n0 = (blockIdx.x * 4 + wave) * (16 * NT);
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_bf16_skinny_kernel(const bf16_t*
                                                                     TO* __restrict__ C, int M, int N, int K) {
   constexpr int WT = GATED ? 2 * NT : NT;  // weight tiles per block
   extern __shared__ float red[];            // [NW][WT][MB][4][64]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = uniform_wave_number();
   const int r16 = lane & 15, quad = lane >> 4;
   const int n0 = blockIdx.x * 16 * NT;
   const bf16_t* wrow[WT];
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(64 * KW * NWV) void gemm_bf16_mid_kernel(const bf16
   static_assert(DEPTH == 1 || DEPTH == 2, "the weights run one or two chunks ahead");
   extern __shared__ __align__(16) unsigned char smem_raw[];  // [KW][2] staged chunks
   const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave = uniform_wave_number();
   const int kg = wave / NWV, nw = wave % NWV;
   const int r16 = lane & 15, quad = lane >> 4;
   const int ntiles = N >> 4;
