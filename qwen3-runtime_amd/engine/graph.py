@@ -13,6 +13,7 @@ a memset node is recorded.
 
 from __future__ import annotations
 
+import gc
 from typing import Sequence
 
 import numpy as np
@@ -185,8 +186,19 @@ class DecodeGraph:
                 # need is that of the largest, not the sum over batch sizes and buckets
                 if runner._graph_pool is None:
                     runner._graph_pool = torch.cuda.graph_pool_handle()
-                with torch.cuda.graph(graph, pool=runner._graph_pool):
-                    self.logits = runner.model.forward(self.ctx, dev["ids"], self.cache_views, dev["rows"])
+                # Graphs of an engine that was dropped earlier may still wait for the collector of
+                # reference cycles; destroying a graph is not allowed while a stream captures, and
+                # the error is raised in a destructor, which ends the process. So collect now, and
+                # keep the collector from running inside the capture.
+                gc.collect()
+                collecting = gc.isenabled()
+                gc.disable()
+                try:
+                    with torch.cuda.graph(graph, pool=runner._graph_pool):
+                        self.logits = runner.model.forward(self.ctx, dev["ids"], self.cache_views, dev["rows"])
+                finally:
+                    if collecting:
+                        gc.enable()
                 self.graph = graph
         runner.last_row_slots = self.views_dev["row_slots"]
         self.graph.replay()

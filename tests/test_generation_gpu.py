@@ -61,6 +61,39 @@ def test_graph_replay_equals_eager(model_folders, dtype):
     assert m.generate(prompts, max_tokens=40) == eager
 
 
+def test_capture_meets_no_garbage_of_an_earlier_engine(model_folders):
+    """An engine with captured graphs, dropped while part of a reference cycle, lives on until the
+    collector of cycles runs. If that happened inside a later engine's capture, the old graphs
+    would be destroyed while a stream captures, which is an error raised in a destructor: the
+    process ends. The capture therefore collects first and keeps the collector out; here the model
+    collects by hand inside the capture, which finds nothing left to destroy."""
+    import gc
+
+    cfg, _ = P.read_model(model_folders["tiny_b"])
+    prompts = prompts_for(cfg, [12, 5], seed=4)
+    first = llm(model_folders["tiny_b"], graph=True)
+    want = first.generate(prompts, max_tokens=8)
+    assert first.engine.runner._graphs
+    cycle = [first]
+    cycle.append(cycle)
+    del first, cycle
+
+    second = llm(model_folders["tiny_b"], graph=True)
+    model = second.engine.runner.model
+    forward, seen = model.forward, []
+
+    def forward_and_collect(*args, **kwargs):
+        if torch.cuda.is_current_stream_capturing():
+            seen.append(gc.isenabled())
+            gc.collect()
+        return forward(*args, **kwargs)
+
+    model.forward = forward_and_collect
+    assert second.generate(prompts, max_tokens=8) == want
+    assert seen and not any(seen), "no capture happened, or the collector was left on inside it"
+    assert gc.isenabled()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replay_across_a_context_bucket(model_folders, dtype):
     """A request that grows past 512 tokens while decoding moves to the graph of the next bucket
