@@ -501,22 +501,28 @@ static int launch_mid(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, 
   return 0;
 }
 
-// 17 to 64 rows on tile-major weights. Configurations from timing a dozen of them on the
-// shapes of the 4B model at 32 and 64 rows: two K groups of two waves with two tiles each where
-// the result is wanted whole; one group of three waves, a gate and an up tile each, for the
-// gated form; one group of three waves with two tiles each where K is cut over blocks.
+// 17 to 64 rows on tile-major weights. Configurations from timing every combination of 1 to 4
+// K groups, 1 to 4 waves a group, 1 or 2 tiles a wave, chunks of 4, 6 or 8 k-steps and weights
+// one or two chunks ahead that fits LDS and registers (some 150 per form) on the shapes of the
+// 4B and 8B models at 32 and 64 rows, each on the weight matrices of 36 layers in turn (one
+// matrix over and over stays in the memory-side cache and flatters every configuration, the
+// small products most): K groups of two waves with one tile each where the result is wanted
+// whole (three groups from 33 rows on, two below: 12.4 us against 13.6 for the former choice
+// at 64 rows of the 4B size, 16.7 against 18.5 at the 8B size); one group of three waves, a
+// gate and an up tile each, for the gated form; one group of three waves with two tiles each
+// where K is cut over blocks. The weights run one chunk ahead everywhere: two chunks lost 3 to
+// 6 % in the gated form.
 template <int MB>
 static int mid(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K, int gated,
                hipStream_t st, int k_parts) {
-  constexpr int DEPTH = MB <= 4 ? 2 : 1;  // more rows: more registers for activations, fewer for the weights' ring
-  if (gated) return launch_mid<MB, 1, 3, 1, 6, DEPTH, true>(a, w, c, out_dtype, M, N, K, st, 1);
+  if (gated) return launch_mid<MB, 1, 3, 1, 6, 1, true>(a, w, c, out_dtype, M, N, K, st, 1);
   if (k_parts > 1) return launch_mid<MB, 1, 3, 2, 6, 1, false>(a, w, c, out_dtype, M, N, K, st, k_parts);
   // The whole result of an ungated product: up to 64 rows only. Beyond, every block would have to
   // fetch more activations than weights, and the vendor library was measured to be faster.
   if constexpr (MB <= 4) {
     // very many tiles (the vocabulary head): eight tiles share the staged activations
     if (N >= 32768) return launch_mid<MB, 1, 4, 2, 8, 1, false>(a, w, c, out_dtype, M, N, K, st, 1);
-    return launch_mid<MB, 2, 2, 2, 4, 2, false>(a, w, c, out_dtype, M, N, K, st, 1);
+    return launch_mid<MB, (MB <= 2 ? 2 : 3), 2, 1, 4, 1, false>(a, w, c, out_dtype, M, N, K, st, 1);
   }
   return qrt_fail("gemm_bf16: above 64 rows only the gated form and products cut along K run on tile-major weights (M=%d)", M);
 }

@@ -167,7 +167,11 @@ class HipOps:
     # instead of the few-row kernel (both stream tile-major weights). Measured at the 4B
     # shapes: cut along K the sharing kernel alone is 5 to 22 % faster from 4 rows on, gated
     # from 12 rows on; a decode step is as fast either way at batch 8 and 5 % faster with it
-    # at batch 16.
+    # at batch 16. (Timed on one weight matrix over and over, the sharing kernel looks 15 to
+    # 40 % faster than the few-row kernel down to one row, because a matrix of up to some
+    # 100 MB then stays in the memory-side cache; with the matrices of 36 layers in turn, as in
+    # a step, it is 5 % slower at 8 rows, and a decode step with it from one row on lost 3 % at
+    # batch 8 and 9 % at batch 1.)
     shared_from_rows = {"whole": 17, "gated": 12, "planes": 9}
     # tiles of 16 rows per wave in the attention kernel for long portions (1 or 2)
     prefill_row_tiles = 2
@@ -384,7 +388,12 @@ class HipOps:
         if not shared:
             if tiles >= 384 or k < 2048:
                 return 1
-            return 2 if k < 8192 else 4
+            # parts of about 1,024 columns, and about a thousand blocks or more in all, in a
+            # number of planes the residual's norm knows when compiling (timed on the matrices of
+            # 36 layers in turn at the 4B, 8B and 32B sizes: 6 to 13 % less than 2 or 4 parts for
+            # the narrow 4B products, level at the 8B size, 1 to 6 % less at the 32B size)
+            want = max(k // 1024, -(-1024 // tiles))
+            return 2 if want <= 2 else 4 if want <= 4 else 8
         blocks = (tiles + 5) // 6
         return max(1, min(8, 256 // blocks, (k // 32) // 12))
 
