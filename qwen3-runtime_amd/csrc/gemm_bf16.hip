@@ -233,15 +233,27 @@ static int skinny(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int 
   return launch_skinny<1, 16, 1, 8, GATED>(a, w, c, out_dtype, M, N, K, st);
 }
 
-// Tile-major weights, M <= 16. Configurations from timing all of them on the shapes of the
-// 4B model: eight waves and eight steps in flight everywhere; two row tiles per block where
-// there are many tiles and no gate (the activations are then read half as often).
+// Tile-major weights, M <= 16. Configurations from timing 78 of them (2 to 16 waves, 1 to 4 row
+// tiles a block, 2 to 12 steps in flight) on the shapes of the 4B, 8B and 32B models at 1 to 16
+// rows, on the weight matrices of 36 layers in turn and replayed from a graph: eight waves
+// everywhere. Gated: one row tile, eight steps in flight (the best at every size). The whole
+// result of a matrix with many row tiles: two tiles a block, so that the activations are read
+// half as often; with two steps in flight up to K = 4,096 (the 8B q/k/v product 10.3 us against
+// 11.8 with eight), with eight for the vocabulary head (7.0 TB/s). K cut into planes: two tiles
+// a block from K = 12,288 on (the 32B down projection at 8 rows 40.4 us against 45.0), four
+// steps in flight up to K = 4,096, eight between.
 template <bool GATED>
 static int skinny_tiled(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K,
                         hipStream_t st, int k_parts) {
   const int tiles = N / 16;
-  if (!GATED && tiles >= 384 && k_parts == 1)
-    return launch_skinny<1, 8, 2, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
+  if (GATED) return launch_skinny<1, 8, 1, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st, k_parts);
+  if (k_parts == 1) {
+    if (tiles >= 2048) return launch_skinny<1, 8, 2, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
+    if (tiles >= 384 && K <= 4096) return launch_skinny<1, 8, 2, 2, GATED, true>(a, w, c, out_dtype, M, N, K, st);
+    return launch_skinny<1, 8, 1, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st);
+  }
+  if (K >= 12288) return launch_skinny<1, 8, 2, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st, k_parts);
+  if (K <= 4096) return launch_skinny<1, 8, 1, 4, GATED, true>(a, w, c, out_dtype, M, N, K, st, k_parts);
   return launch_skinny<1, 8, 1, 8, GATED, true>(a, w, c, out_dtype, M, N, K, st, k_parts);
 }
 
