@@ -67,6 +67,18 @@ struct AttnTileArgs {
   // the tokens whose rows the merge of key splits may write; null: all rows
   const int* merge_tokens;
   int num_merge_tokens;
+  // Decoding with the step's own keys and values still in the product that made them (one
+  // token per sequence; qkv non-null): the kernel normalises and rotates the token's query and
+  // key heads itself, attends over the cache up to the token before, adds the token's own key
+  // and value from registers, and stores them into the cache for the steps to come. `q` is
+  // then unused.
+  const bf16_t* qkv;       // [T, qkv_stride]: nq query heads, nkv key heads, nkv value heads of D
+  long qkv_stride;
+  const float* q_weight;   // [D] or null: no norm
+  const float* k_weight;
+  const float* rope;       // [T, D]: cosines of the D / 2 angles, then their sines; null: no rotation
+  const int* slots;        // [T]: place of the token in the cache, page * page_size + offset
+  float eps;
 };
 
 constexpr int D = QRT_HEAD_DIM;
@@ -696,9 +708,57 @@ __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg
   tile_update(s, blk.v, !whole, base, quad, row_valid, qpos, window, scale_log2, m, l, o);
 }
 
+// One head of a token's product (x, D elements, D a multiple of 64) as an MFMA operand: RMSNorm
+// over the head in float32 (weight after the normalisation), NeoX rotation pairing element j
+// with j + D / 2 by the angles of `rope`, rounded to bfloat16 last, as the kernel that writes
+// queries and keys to memory does. A lane holds elements 32 i + 8 quad .. + 7 of k-step i, so a
+// pair lies in one lane (k-steps i and i + KFULL / 2) and the head's sum of squares in the four
+// lanes of a row.
+__device__ __forceinline__ void head_as_operand(const bf16_t* __restrict__ x, const float* __restrict__ w,
+                                                const float* __restrict__ rope, float eps, int quad,
+                                                bf16x8_t* out) {
+  constexpr int KF = KFULL > 0 ? KFULL : 1, HALF_STEPS = KF / 2;
+  float v[KF][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < KF; ++i) {
+    const bf16x8_t r = *(const bf16x8_t*)(x + 32 * i + 8 * quad);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[i][e] = (float)r[e];
+      ss += v[i][e] * v[i][e];
+    }
+  }
+  if (w) {
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    const float inv = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int i = 0; i < KF; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[i][e] = v[i][e] * inv * w[32 * i + 8 * quad + e];
+  }
+  if (rope) {
+#pragma unroll
+    for (int i = 0; i < HALF_STEPS; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = 32 * i + 8 * quad + e;
+        const float cs = rope[j], sn = rope[D / 2 + j];
+        const float x1 = v[i][e], x2 = v[i + HALF_STEPS][e];
+        v[i][e] = x1 * cs - x2 * sn;
+        v[i + HALF_STEPS][e] = x2 * cs + x1 * sn;
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < KF; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[i][e] = (bf16_t)v[i][e];
+}
+
 constexpr bool DECODE_ONCE = true;  // measured: 2 % off a decode step at batch 1 and at batch 64, level at batch 8
 
-template <bool P2>
+template <bool P2, bool FUSED = false>
 __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_decode_kernel(AttnTileArgs a) {
   // per wave: maximum and sum per row, unnormalised accumulator [16][D]
   extern __shared__ float lds[];
@@ -731,21 +791,73 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
   for (int i = 0; i < DB; ++i) o[i] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  const int pos_min = first_pos, pos_max = first_pos + (max(n_rows, 1) - 1) / g;
-  const int lo = a.window > 0 ? max(0, pos_min - a.window + 1) : 0;
-  const int blk_begin = lo >> 5, blk_end = (pos_max >> 5) + 1;
+  // FUSED (one token per sequence, at position first_pos): the cache holds the keys before it,
+  // [lo, first_pos - 1]; the token itself is added from registers below. For the masks of the
+  // cache's blocks the token then stands one position earlier with a window one shorter.
+  const int own = FUSED ? 1 : 0;
+  const int window = FUSED && a.window > 0 ? a.window - 1 : a.window;
+  const int qpos_c = qpos - own;
+  const int pos_min = first_pos - own, pos_max = first_pos + (max(n_rows, 1) - 1) / g - own;
+  const int lo = a.window > 0 ? max(0, first_pos - a.window + 1) : 0;
+  const bool any_cached = !FUSED || (pos_max >= lo && a.window != 1);
+  const int blk_begin = lo >> 5, blk_end = any_cached ? (pos_max >> 5) + 1 : blk_begin;
   const int per = (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
   const int b0 = blk_begin + split * per;
   const int b1 = min(blk_end, b0 + per);
   int b = b0 + wave;
 
-  if (n_rows > 0 && b < b1) {
-    const bf16_t* qp = a.q + ((size_t)(q_begin + tok) * a.nq + head) * D;
-    bf16x8_t qreg[KFULL > 0 ? KFULL : 1];
+  bf16x8_t qreg[KFULL > 0 ? KFULL : 1];
+  bf16x8_t qtail = load_tail((const bf16_t*)nullptr, 2);  // zeros
+  if (FUSED) {
+    // every wave forms the queries it multiplies; the first wave of the first split also takes
+    // the token's own key and value, the second wave stores them into the cache
+    const bf16_t* raw = a.qkv + (size_t)q_begin * a.qkv_stride;
+    const float* rope = a.rope ? a.rope + (size_t)q_begin * D : nullptr;
+    head_as_operand(raw + (size_t)head * D, a.q_weight, rope, a.eps, quad, qreg);
+    const bool adds_own = split == 0 && wave == 0, stores_own = split == 0 && wave == 1 % DW;
+    if (adds_own || stores_own) {  // uniform over the wave
+      const bf16_t* kraw = raw + ((size_t)a.nq + kvh) * D;
+      const bf16_t* vraw = raw + ((size_t)a.nq + a.nkv + kvh) * D;
+      bf16x8_t kreg[KFULL > 0 ? KFULL : 1];
+      head_as_operand(kraw, a.k_weight, rope, a.eps, quad, kreg);
+      if (stores_own) {
+        const int slot = a.slots[q_begin];
+        const int page = slot / a.page_size, off = slot - page * a.page_size;
+        bf16_t* kdst = (bf16_t*)a.k_cache + (((size_t)page * a.nkv + kvh) * a.page_size + off) * D;
+        bf16_t* vdst = (bf16_t*)a.v_cache + ((size_t)page * a.nkv + kvh) * D * a.page_size + off;
+        if (r16 == 0) {
 #pragma unroll
-    for (int i = 0; i < KFULL; ++i) qreg[i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
-    bf16x8_t qtail = load_tail(qp, 2);  // zeros
-    if (KTAIL) qtail = load_tail(qp + 32 * KFULL, quad);
+          for (int i = 0; i < KFULL; ++i) *(bf16x8_t*)(kdst + 32 * i + 8 * quad) = kreg[i];
+        }
+        for (int d = lane; d < D; d += 64) vdst[(size_t)d * a.page_size] = vraw[d];
+      }
+      if (adds_own) {
+        // a block of keys that holds this one key, in the place of key first_pos: operand row 0
+        // of the first half block; the other rows are masked like keys after the token
+        f32x4_t sc[2];
+        sc[0] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        sc[1] = sc[0];
+#pragma unroll
+        for (int i = 0; i < KFULL; ++i) sc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[i], qreg[i], sc[0], 0, 0, 0);
+        bf16x8_t vv[DB];
+#pragma unroll
+        for (int i = 0; i < DB; ++i) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) vv[i][e] = (bf16_t)0.0f;
+          if (quad == 0) vv[i][0] = vraw[16 * i + r16];
+        }
+        tile_update(sc, vv, true, first_pos, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+      }
+    }
+  }
+
+  if (n_rows > 0 && b < b1) {
+    if (!FUSED) {
+      const bf16_t* qp = a.q + ((size_t)(q_begin + tok) * a.nq + head) * D;
+#pragma unroll
+      for (int i = 0; i < KFULL; ++i) qreg[i] = *(const bf16x8_t*)(qp + 32 * i + 8 * quad);
+      if (KTAIL) qtail = load_tail(qp + 32 * KFULL, quad);
+    }
 
     // keys and values are loaded one block ahead, page numbers two; past the wave's last block
     // the loads repeat that block (their data is not used)
@@ -758,12 +870,12 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
     while (true) {
       block_load<P2, DECODE_ONCE>(a, kvh, min(b + DW, last) << 5, lo, pos_max, r16, quad, pgB, B);
       block_pages<P2>(table, min(b + 2 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
-      block_compute(A, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+      block_compute(A, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.scale_log2, m, l, o);
       b += DW;
       if (b >= b1) break;
       block_load<P2, DECODE_ONCE>(a, kvh, min(b + DW, last) << 5, lo, pos_max, r16, quad, pgA, A);
       block_pages<P2>(table, min(b + 2 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
-      block_compute(B, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
+      block_compute(B, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.scale_log2, m, l, o);
       b += DW;
       if (b >= b1) break;
     }
@@ -837,7 +949,30 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
       allowed = true;
     }
   }
-  if (p2) attention_bf16_decode_kernel<true><<<grid, block, smem, stream>>>(a);
+  if (a.qkv) {
+    // one token per sequence, its query, key and value taken from the product that made them
+    if constexpr (D % 64 == 0) {
+      QRT_CHECK(a.nq / a.nkv <= 16 && a.slots && a.qkv_stride >= (long)(a.nq + 2 * a.nkv) * D && a.qkv_stride % 8 == 0 &&
+                    (uintptr_t)a.qkv % 16 == 0,
+                "attention (decode, own token from the product): %d query heads per key head, stride %ld",
+                a.nq / a.nkv, a.qkv_stride);
+      if (smem > 64 * 1024) {
+        static bool allowed_fused = false;
+        if (!allowed_fused) {
+          if (hipFuncSetAttribute((const void*)attention_bf16_decode_kernel<true, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess ||
+              hipFuncSetAttribute((const void*)attention_bf16_decode_kernel<false, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+            return qrt_fail("attention (decode): cannot get %zu bytes of LDS", smem);
+          allowed_fused = true;
+        }
+      }
+      if (p2) attention_bf16_decode_kernel<true, true><<<grid, block, smem, stream>>>(a);
+      else attention_bf16_decode_kernel<false, true><<<grid, block, smem, stream>>>(a);
+    } else {
+      return qrt_fail("attention (decode, own token from the product): head size %d is no multiple of 64", D);
+    }
+  } else if (p2) attention_bf16_decode_kernel<true><<<grid, block, smem, stream>>>(a);
   else attention_bf16_decode_kernel<false><<<grid, block, smem, stream>>>(a);
   QRT_LAUNCH_CHECK("attention_bf16_decode");
   if (a.num_splits > 1) {

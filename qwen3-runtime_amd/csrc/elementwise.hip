@@ -31,6 +31,31 @@ extern "C" int qrt_embed(const int* ids, const void* table, int table_dtype, flo
   return 0;
 }
 
+// ------------------------------------------------ rotation table of a step
+// out[t, j] = cos(pos[t] * inv_freq[j]), out[t, half + j] = sin(...), j < half: the angles of a
+// step's tokens, float32. Every layer of a step rotates by the same angles, so a step that
+// rotates inside its attention kernel computes them once, here, and the layers look them up.
+__global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  float* __restrict__ out, int half) {
+  const float pos = (float)positions[blockIdx.x];
+  float* row = out + (size_t)blockIdx.x * 2 * half;
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    float sn, cs;
+    sincos_angle(pos * inv_freq[j], &sn, &cs);
+    row[j] = cs;
+    row[half + j] = sn;
+  }
+}
+
+extern "C" int qrt_rope_table(const int* positions, const float* inv_freq, float* out, int num_tokens, int half,
+                              hipStream_t stream) {
+  QRT_CHECK(num_tokens >= 0 && half > 0, "rope_table: bad sizes T=%d half=%d", num_tokens, half);
+  if (num_tokens == 0) return 0;
+  rope_table_kernel<<<dim3(num_tokens), dim3(half <= 64 ? 64 : 128), 0, stream>>>(positions, inv_freq, out, half);
+  QRT_LAUNCH_CHECK("rope_table");
+  return 0;
+}
+
 // ------------------------------------------------------- add + RMSNorm
 // r = rows ? rows[b] : b
 // x = residual[r] (+ delta[r]);  without `rows` the sum is written back.

@@ -66,6 +66,8 @@ class _AttnTileArgs(Structure):
         ("page_size", c_int), ("window", c_int), ("num_splits", c_int), ("waves", c_int),
         ("scale_log2", c_float), ("row_tiles", c_int), ("use_lds", c_int),
         ("merge_tokens", c_void_p), ("num_merge_tokens", c_int),
+        ("qkv", c_void_p), ("qkv_stride", c_long), ("q_weight", c_void_p), ("k_weight", c_void_p),
+        ("rope", c_void_p), ("slots", c_void_p), ("eps", c_float),
     ]
 
 
@@ -173,6 +175,8 @@ class HipOps:
     # a step, it is 5 % slower at 8 rows, and a decode step with it from one row on lost 3 % at
     # batch 8 and 9 % at batch 1.)
     shared_from_rows = {"whole": 17, "gated": 12, "planes": 9}
+    # steps of single tokens: norm, rotation, cache write and attention in one kernel
+    fuse_decode = True
     # tiles of 16 rows per wave in the attention kernel for long portions (1 or 2)
     prefill_row_tiles = 2
     # long portions: keys and values go through LDS, shared by the four waves of a block
@@ -510,6 +514,59 @@ class HipOps:
         return pages
 
     # ---- attention ---------------------------------------------------------------
+    # ---- decoding: norm, rotation, cache write and attention in one kernel -------------
+    def rope_table(self, ctx, inv_freq):
+        """Cosines and sines of the step's rotation angles, float32 [T, 2 * len(inv_freq)]
+        (cosines first): computed once per step and looked up by every layer that rotates inside
+        its attention kernel."""
+        key = ("rope_table", inv_freq.data_ptr())
+        table = ctx.per_pass.get(key)
+        if table is None:
+            half = inv_freq.numel()
+            _need(inv_freq, "inv_freq", torch.float32, (half,))
+            _need(ctx.positions, "positions", torch.int32, (ctx.num_tokens,))
+            table = torch.empty((ctx.num_tokens, 2 * half), dtype=torch.float32, device=inv_freq.device)
+            self._check(self.lib, self.lib.qrt_rope_table(_ptr(ctx.positions), _ptr(inv_freq), _ptr(table),
+                                                          c_int(ctx.num_tokens), c_int(half), _stream()))
+            ctx.per_pass[key] = table
+        return table
+
+    def fuses_decode_attention(self, ctx, qkv, nq, nkv, d, cache) -> bool:
+        """Whether ``decode_attention`` serves this step: one token per sequence, bfloat16, a head
+        size that keeps a rotation pair in one lane (a multiple of 64, up to 256), at most 16
+        query heads per key head, and a layer that writes its own cache."""
+        return (self.fuse_decode and qkv.dtype == torch.bfloat16 and ctx.max_q_len == 1
+                and ctx.num_tokens == ctx.num_seqs and d % 64 == 0 and d <= 256 and nq // nkv <= 16
+                and cache is not None and cache.writes and cache.group.page_size % 8 == 0
+                and cache.k.dtype == torch.bfloat16)
+
+    def decode_attention(self, qkv, cache, ctx, nq, nkv, d, scale, window, q_w, k_w, eps, inv_freq):
+        """``paged_attention(qk_norm_rope_store(qkv, ...))`` for a step of single tokens, in one
+        kernel: each block forms its queries from ``qkv`` (RMSNorm per head, NeoX rotation by the
+        step's angle table), attends over the cached keys before the token, adds the token's own
+        key and value from registers and stores them into the cache for later steps. Saves the
+        kernel between the product and the attention, and the round trip of the queries."""
+        t, width = qkv.shape
+        _need(qkv, "qkv", torch.bfloat16, (t, (nq + 2 * nkv) * d))
+        self._check_cache(cache, nkv, d, qkv.dtype)
+        for name, w in (("q_norm", q_w), ("k_norm", k_w)):
+            if w is not None:
+                _need(w, name, torch.float32, (d,))
+        _need(cache.group.slots, "slots", torch.int32, (t,))
+        table = _need(cache.group.block_table, "block table", torch.int32)
+        if table.shape[0] != ctx.num_seqs:
+            raise OpsError(f"block table has {table.shape[0]} rows for {ctx.num_seqs} sequences")
+        ps = cache.group.page_size
+        if table.shape[1] < (ctx.max_kv_len + ps - 1) // ps:
+            raise OpsError(f"block table is {table.shape[1]} pages wide, the longest sequence needs more")
+        if not scale > 0:
+            raise OpsError(f"the bfloat16 attention kernels take a positive score scale, not {scale}")
+        own = {"qkv": qkv, "q_weight": q_w, "k_weight": k_w, "eps": eps,
+               "rope": None if inv_freq is None else self.rope_table(ctx, inv_freq)}
+        out = torch.empty((t, nq * d), dtype=qkv.dtype, device=qkv.device)
+        self._launch_attention(None, out, cache, ctx, nq, nkv, d, scale, window or 0, None, True, own)
+        return out
+
     def paged_attention(self, q, cache, ctx, nq, nkv, d, scale, window):
         t = ctx.num_tokens
         _need(q, "q", shape=(t, nq * d))
@@ -603,7 +660,7 @@ class HipOps:
             return
         self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False)
 
-    def _launch_attention(self, q, out, cache, ctx, nq, nkv, d, scale, window, subset, decode):
+    def _launch_attention(self, q, out, cache, ctx, nq, nkv, d, scale, window, subset, decode, own=None):
         """One launch over the sequences in ``subset`` (None: all of the step's)."""
         lib = attention_library(d)
         g = nq // nkv
@@ -622,7 +679,7 @@ class HipOps:
         key = ("attn_plan", g, nkv, d, waves, row_tiles, decode, None if subset is None else tuple(subset))
         plan = ctx.scratch.get(key)
         if plan is None:  # the same for every layer of the step
-            dev = q.device
+            dev = out.device
             if decode:
                 tiles = None if subset is None else torch.tensor(subset, dtype=torch.int32, device=dev)
                 n_tiles = len(q_lens)
@@ -642,7 +699,13 @@ class HipOps:
         splits = ctx.scratch.get("attn_splits") or (
             self.choose_decode_splits(n_tiles, nkv, max_kv) if decode else self.choose_splits(n_tiles, nkv, max_kv))
         a = _AttnTileArgs()
-        a.q, a.out, a.k_cache, a.v_cache = q.data_ptr(), out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
+        a.out, a.k_cache, a.v_cache = out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
+        if own is None:
+            a.q = q.data_ptr()
+        else:  # the token's own query, key and value come from the product that made them
+            a.qkv, a.qkv_stride = own["qkv"].data_ptr(), own["qkv"].shape[1]
+            a.q_weight, a.k_weight, a.rope = _addr(own["q_weight"]), _addr(own["k_weight"]), _addr(own["rope"])
+            a.slots, a.eps = cache.group.slots.data_ptr(), own["eps"]
         a.cu_q = _need(ctx.cu_q, "cu_q", torch.int32, (ctx.num_seqs + 1,)).data_ptr()
         a.kv_lens = _need(ctx.kv_lens, "kv_lens", torch.int32, (ctx.num_seqs,)).data_ptr()
         a.block_table, a.table_width = cache.group.block_table.data_ptr(), cache.group.block_table.shape[1]
@@ -657,8 +720,8 @@ class HipOps:
         a.use_lds = 1 if self.prefill_through_lds else 0
         a.scale_log2 = scale * math.log2(math.e)
         if splits > 1:
-            part_o = torch.empty((ctx.num_tokens * nq * splits, d), dtype=torch.float32, device=q.device)
-            part_lse = torch.empty((ctx.num_tokens * nq * splits,), dtype=torch.float32, device=q.device)
+            part_o = torch.empty((ctx.num_tokens * nq * splits, d), dtype=torch.float32, device=out.device)
+            part_lse = torch.empty((ctx.num_tokens * nq * splits,), dtype=torch.float32, device=out.device)
             a.part_o, a.part_lse = part_o.data_ptr(), part_lse.data_ptr()
         if decode:
             self._check(lib, lib.qrt_attention_bf16_decode(byref(a), c_int(ctx.num_tokens * nq), _stream()))

@@ -84,9 +84,14 @@ class GroupedQueryAttention(Mixer):
         qkv = ops.linear(x, self.qkv)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
         fused = self.position is None or self.position.fused_form == "neox_full"
+        inv_freq = None if self.position is None or not fused else self.position.inv_freq
+        if fused and ops.fuses_decode_attention(ctx, qkv, nq, nkv, d, cache):
+            # a step of single tokens: all of it inside the attention kernel
+            attn = ops.decode_attention(qkv, cache, ctx, nq, nkv, d, self.scale, self.window,
+                                        self.q_norm, self.k_norm, eps, inv_freq)
+            return ops.linear_for_residual(attn, self.o)
         if fused:
             # norm, rotation and the cache write in one pass over qkv
-            inv_freq = None if self.position is None else self.position.inv_freq
             q = ops.qk_norm_rope_store(
                 qkv, nq, nkv, d, self.q_norm, self.k_norm, eps, inv_freq, ctx.positions,
                 cache if cache.writes else None,

@@ -166,3 +166,7 @@ class StepContext:
     max_kv_len: int = 0
     groups: list[GroupView] = field(default_factory=list)
     scratch: dict[str, Any] = field(default_factory=dict)
+    # values computed from the step's own data (positions, lengths) that several layers share: the
+    # model empties this at the start of every pass, also of one that reuses the context (a
+    # captured graph keeps its context, and what is computed here must be part of the capture)
+    per_pass: dict[Any, Any] = field(default_factory=dict)

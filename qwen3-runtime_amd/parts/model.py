@@ -99,6 +99,7 @@ class DecoderModel:
         (int32 tensor), or None when ``rows`` is None: the pass then only fills
         the caches.
         """
+        ctx.per_pass.clear()
         residual = self.embedding.forward(ctx, ids)
         delta = None
         for step, cache in zip(self.plan.order, caches):

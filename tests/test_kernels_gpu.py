@@ -442,6 +442,59 @@ def test_paged_attention_window(ops, dtype, window):
     close(got, want, tol, tol)
 
 
+@pytest.mark.parametrize("nq,nkv,d,ps,window,norm,rope", [
+    (32, 8, 128, 16, None, True, True),     # the 4B geometry
+    (8, 2, 64, 16, None, True, True),
+    (5, 1, 128, 24, None, True, True),      # five query heads per key head, pages of 24
+    (16, 1, 64, 8, None, True, False),      # sixteen rows: no row to spare; no rotation
+    (4, 4, 256, 16, None, False, True),     # one query head per key head, head size 256, no norm
+    (6, 2, 192, 32, None, True, True),
+    (8, 2, 64, 16, 40, True, True),         # a window over the cache and the token itself
+    (8, 2, 128, 8, 1, True, True),          # a window of the token alone
+])
+def test_decode_attention_with_the_tokens_own_key_from_the_product(ops, nq, nkv, d, ps, window, norm, rope):
+    """A step of single tokens in one kernel: queries and the token's key normalised and rotated
+    inside the attention kernel, the token's key and value added from registers and stored into
+    the cache. Against the plain norm-rotate-store followed by the plain attention: the output,
+    the cache at the tokens' places, and the cache everywhere else (untouched). The tokens' places
+    hold stale noise beforehand, which must not be read; contexts of 1 (no cached key at all) to
+    2,100 keys (several key splits), ends of blocks of 32 and of pages."""
+    kvs = [1, 2, 32, 33, 64, 65, 300, 2100, ps, ps + 1]
+    seqs = [(1, kv) for kv in kvs]
+    _, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, window=window, seed=3)
+    t = len(seqs)
+    qkv = rnd(t, (nq + 2 * nkv) * d, dtype=torch.bfloat16, seed=11)
+    qw = 1 + 0.1 * rnd(d, seed=5) if norm else None
+    kw = 1 + 0.1 * rnd(d, seed=6) if norm else None
+    inv = (1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV) if rope else None
+    table = cache.group.block_table.cpu()
+    slots = torch.tensor([int(table[i, (kv - 1) // ps]) * ps + (kv - 1) % ps for i, kv in enumerate(kvs)],
+                         dtype=torch.int32, device=DEV)
+    cache.group.slots = slots
+    scale = 1.0 / math.sqrt(d)
+    want_k, want_v = cache.k.clone(), cache.v.clone()
+    q = R.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, ctx.positions, want_k, want_v, slots, ps)
+    want = R.paged_attention(q.to(torch.bfloat16), want_k, want_v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(),
+                             cache.group.block_table, ps, nq, nkv, d, scale, window)
+    before_k, before_v = cache.k.clone(), cache.v.clone()
+    assert ops.fuses_decode_attention(ctx, qkv, nq, nkv, d, cache)
+    got = ops.decode_attention(qkv, cache, ctx, nq, nkv, d, scale, window, qw, kw, 1e-6, inv)
+    close(got, want, 2e-2, 2e-2)
+    # the cache: the tokens' own places as the plain store leaves them, all else as before
+    changed_k = (want_k != before_k)
+    changed_v = (want_v != before_v)
+    close(cache.k[changed_k], want_k[changed_k], 2e-2, 2e-2)
+    close(cache.v[changed_v], want_v[changed_v], 0, 0)
+    assert torch.equal(cache.k[~changed_k], before_k[~changed_k])
+    assert torch.equal(cache.v[~changed_v], before_v[~changed_v])
+    # with the keys cut over other numbers of blocks
+    for splits in (1, 3, 16):
+        cache.k.copy_(before_k)
+        cache.v.copy_(before_v)
+        ctx.scratch["attn_splits"] = splits
+        close(ops.decode_attention(qkv, cache, ctx, nq, nkv, d, scale, window, qw, kw, 1e-6, inv), want, 2e-2, 2e-2)
+
+
 def test_paged_attention_splits_agree(ops):
     """Long single sequences split over many blocks; empty splits must not leak."""
     seqs, nq, nkv, d, ps = [(1, 2100), (1, 40), (3, 900)], 8, 2, 64, 16
