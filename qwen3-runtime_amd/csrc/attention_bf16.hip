@@ -808,13 +808,16 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
 
   bf16x8_t qreg[KFULL > 0 ? KFULL : 1];
   bf16x8_t qtail = load_tail((const bf16_t*)nullptr, 2);  // zeros
-  if (FUSED) {
-    // every wave forms the queries it multiplies; the first wave of the first split also takes
-    // the token's own key and value, the second wave stores them into the cache
+  // every wave forms the queries it multiplies; the last wave of the last split also takes the
+  // token's own key and value, the wave before it stores them into the cache (these have the
+  // fewest blocks of cached keys: the blocks go round the waves, and the last split takes what
+  // the others left)
+  auto own_token = [&]() {
     const bf16_t* raw = a.qkv + (size_t)q_begin * a.qkv_stride;
     const float* rope = a.rope ? a.rope + (size_t)q_begin * D : nullptr;
     head_as_operand(raw + (size_t)head * D, a.q_weight, rope, a.eps, quad, qreg);
-    const bool adds_own = split == 0 && wave == 0, stores_own = split == 0 && wave == 1 % DW;
+    const bool at_end = split == (int)gridDim.z - 1;
+    const bool adds_own = at_end && wave == DW - 1, stores_own = at_end && wave == (2 * DW - 2) % DW;
     if (adds_own || stores_own) {  // uniform over the wave
       const bf16_t* kraw = raw + ((size_t)a.nq + kvh) * D;
       const bf16_t* vraw = raw + ((size_t)a.nq + a.nkv + kvh) * D;
@@ -849,7 +852,7 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
         tile_update(sc, vv, true, first_pos, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
       }
     }
-  }
+  };
 
   if (n_rows > 0 && b < b1) {
     if (!FUSED) {
@@ -867,6 +870,7 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
     block_pages<P2>(table, b << 5, lo, pos_max, a.page_size, r16, quad, pgA);
     block_pages<P2>(table, min(b + DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
     block_load<P2, DECODE_ONCE>(a, kvh, b << 5, lo, pos_max, r16, quad, pgA, A);
+    if (FUSED) own_token();  // while the first keys and values are on their way
     while (true) {
       block_load<P2, DECODE_ONCE>(a, kvh, min(b + DW, last) << 5, lo, pos_max, r16, quad, pgB, B);
       block_pages<P2>(table, min(b + 2 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
@@ -879,6 +883,8 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
       b += DW;
       if (b >= b1) break;
     }
+  } else if (FUSED) {
+    own_token();
   }
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);

@@ -515,11 +515,12 @@ class HipOps:
 
     # ---- attention ---------------------------------------------------------------
     # ---- decoding: norm, rotation, cache write and attention in one kernel -------------
-    def rope_table(self, ctx, inv_freq):
+    def rope_table(self, ctx, inv_freq, angles_key=None):
         """Cosines and sines of the step's rotation angles, float32 [T, 2 * len(inv_freq)]
-        (cosines first): computed once per step and looked up by every layer that rotates inside
-        its attention kernel."""
-        key = ("rope_table", inv_freq.data_ptr())
+        (cosines first): computed once per pass and looked up by every layer that rotates inside
+        its attention kernel. ``angles_key`` names the angles (layers with equal keys share the
+        table); without it the tensor ``inv_freq`` itself does."""
+        key = ("rope_table", angles_key if angles_key is not None else inv_freq.data_ptr())
         table = ctx.per_pass.get(key)
         if table is None:
             half = inv_freq.numel()
@@ -540,7 +541,8 @@ class HipOps:
                 and cache is not None and cache.writes and cache.group.page_size % 8 == 0
                 and cache.k.dtype == torch.bfloat16)
 
-    def decode_attention(self, qkv, cache, ctx, nq, nkv, d, scale, window, q_w, k_w, eps, inv_freq):
+    def decode_attention(self, qkv, cache, ctx, nq, nkv, d, scale, window, q_w, k_w, eps, inv_freq,
+                         angles_key=None):
         """``paged_attention(qk_norm_rope_store(qkv, ...))`` for a step of single tokens, in one
         kernel: each block forms its queries from ``qkv`` (RMSNorm per head, NeoX rotation by the
         step's angle table), attends over the cached keys before the token, adds the token's own
@@ -562,7 +564,7 @@ class HipOps:
         if not scale > 0:
             raise OpsError(f"the bfloat16 attention kernels take a positive score scale, not {scale}")
         own = {"qkv": qkv, "q_weight": q_w, "k_weight": k_w, "eps": eps,
-               "rope": None if inv_freq is None else self.rope_table(ctx, inv_freq)}
+               "rope": None if inv_freq is None else self.rope_table(ctx, inv_freq, angles_key)}
         out = torch.empty((t, nq * d), dtype=qkv.dtype, device=qkv.device)
         self._launch_attention(None, out, cache, ctx, nq, nkv, d, scale, window or 0, None, True, own)
         return out

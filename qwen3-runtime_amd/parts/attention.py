@@ -88,7 +88,8 @@ class GroupedQueryAttention(Mixer):
         if fused and ops.fuses_decode_attention(ctx, qkv, nq, nkv, d, cache):
             # a step of single tokens: all of it inside the attention kernel
             attn = ops.decode_attention(qkv, cache, ctx, nq, nkv, d, self.scale, self.window,
-                                        self.q_norm, self.k_norm, eps, inv_freq)
+                                        self.q_norm, self.k_norm, eps, inv_freq,
+                                        None if self.position is None else self.position.angles_key)
             return ops.linear_for_residual(attn, self.o)
         if fused:
             # norm, rotation and the cache write in one pass over qkv

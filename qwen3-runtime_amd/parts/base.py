@@ -103,6 +103,9 @@ class PositionEncoding(Part):
     # half, by the angles ``position * self.inv_freq[j]`` (float32 [head_dim / 2] on the device).
     # None (the default) means the mixer norms, calls ``rotate`` and stores, as three steps.
     fused_form: str | None = None
+    # Encodings with equal keys rotate by equal angles: the layers of a step then share one table
+    # of its tokens' cosines and sines. None: the encoding's own ``inv_freq`` tensor is the key.
+    angles_key: Any = None
 
 
 class Block(Part):

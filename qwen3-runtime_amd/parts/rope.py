@@ -31,6 +31,8 @@ class RotaryNeox(PositionEncoding):
             self.theta ** (torch.arange(0, self.head_dim, 2, dtype=torch.float32) / self.head_dim)
         )
         self.inv_freq = None
+        # layers whose encodings have equal keys rotate by equal angles and share a step's table
+        self.angles_key = ("rope_neox", self.head_dim, self.theta)
 
     def load(self, fetch):
         self.inv_freq = fetch.constant(self.inv_freq_cpu)
