@@ -172,6 +172,9 @@ class TorchOps:
         return qk_norm_rope_store(qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions,
                                   cache.k, cache.v, cache.group.slots, cache.group.page_size, self.compute)
 
+    def fuses_decode_attention(self, ctx, qkv, nq, nkv, d, cache):
+        return False  # no one-kernel form of a decode step's attention here: the steps above, in order
+
     def qk_norm_split(self, qkv, nq, nkv, d, q_w, k_w, eps):
         return qk_norm_split(qkv, nq, nkv, d, q_w, k_w, eps, self.compute)
 
