@@ -61,12 +61,12 @@ def test_graph_replay_equals_eager(model_folders, dtype):
     assert m.generate(prompts, max_tokens=40) == eager
 
 
-def test_capture_meets_no_garbage_of_an_earlier_engine(model_folders):
+def test_the_collector_stays_out_of_a_capture(model_folders):
     """An engine with captured graphs, dropped while part of a reference cycle, lives on until the
     collector of cycles runs. If that happened inside a later engine's capture, the old graphs
     would be destroyed while a stream captures, which is an error raised in a destructor: the
-    process ends. The capture therefore collects first and keeps the collector out; here the model
-    collects by hand inside the capture, which finds nothing left to destroy."""
+    process ends. So the collector is switched off inside every capture (and on again after);
+    the garbage goes at the next collection outside one, here by hand at the end."""
     import gc
 
     cfg, _ = P.read_model(model_folders["tiny_b"])
@@ -85,13 +85,14 @@ def test_capture_meets_no_garbage_of_an_earlier_engine(model_folders):
     def forward_and_collect(*args, **kwargs):
         if torch.cuda.is_current_stream_capturing():
             seen.append(gc.isenabled())
-            gc.collect()
         return forward(*args, **kwargs)
 
     model.forward = forward_and_collect
     assert second.generate(prompts, max_tokens=8) == want
     assert seen and not any(seen), "no capture happened, or the collector was left on inside it"
     assert gc.isenabled()
+    gc.collect()  # the first engine's graphs go now, outside any capture
+    assert second.generate(prompts, max_tokens=8) == want
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
