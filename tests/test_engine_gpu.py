@@ -103,6 +103,48 @@ def test_mixed_with_page_reuse(model_folders, tiny_configs, name, dtype):
     check(got, traces.plain_logits(model_folders[name], reqs), dtype)
 
 
+@pytest.mark.parametrize("seed", [3, 5, 6, 17, 26, 45])
+def test_random_models_and_random_traces(tmp_path, seed):
+    """A model and a trace drawn from the seed: head sizes 16 to 256 (64 and up also take the decode
+    kernel that forms its own queries and keys), 1 to 4 key heads with 1 to 16 query heads each,
+    widths and vocabularies that are multiples of nothing much, pages of 8 to 64, prompts of 1 to
+    1,500 tokens cut at random beside decoded tokens, a pool of exactly the pages the live requests
+    hold at the peak. In float32 and in bfloat16, with and without graphs, against the plain model.
+    (Hundreds of further seeds of this generator were run once; these six are kept.)"""
+    import random
+
+    from qwen3_runtime_amd.config.model import Qwen3Config
+    from qwen3_runtime_amd.weights import write_model_folder
+
+    rng = random.Random(seed)
+    d = rng.choice((16, 48, 64, 64, 128, 128, 192, 256))
+    nkv, g = rng.choice((1, 2, 3, 4)), rng.choice((1, 2, 4, 5, 8, 16))
+    cfg = Qwen3Config(vocab_size=rng.choice((257, 512, 1000)), hidden_size=rng.choice((96, 160, 256, 264)),
+                      num_hidden_layers=rng.choice((1, 2, 3)), num_attention_heads=nkv * g, num_key_value_heads=nkv,
+                      head_dim=d, intermediate_size=rng.choice((128, 208, 512)), rms_norm_eps=rng.choice((1e-6, 1e-5)),
+                      rope_theta=rng.choice((10000.0, 1e6)), max_position_embeddings=4096,
+                      tie_word_embeddings=rng.random() < 0.5)
+    page = rng.choice((8, 16, 16, 24, 32, 64))
+    lengths = [rng.choice((1, 2, 5, 33, 64, 65, 127, 200, 400, 700, 1100, 1500)) for _ in range(rng.randint(2, 6))]
+    write_model_folder(tmp_path, cfg.to_dict(), seed=seed)
+    reqs = traces.make_requests(cfg.vocab_size, lengths, seed=seed)
+    steps = traces.random_trace(reqs, rng, rng.randint(1, 4))
+    pages = traces.peak_tokens(steps, unit=page) // page
+    want = None
+    for dtype in ("float32", "bfloat16"):
+        loaded = load_gpu(tmp_path, page, pages, dtype, hip_graph=rng.random() < 0.5)
+        got = traces.replay(loaded, steps)
+        if want is None:
+            full = traces.plain_logits(tmp_path, reqs)
+            want = {k: full[k] for k in got}
+        if dtype == "float32":
+            traces.compare(got, want, atol=1e-4, rtol=1e-4)
+        else:
+            traces.compare_rounding_noise(got, want)
+        del loaded
+        torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(model_folders, tiny_configs, dtype):
     """A short prompt, then 400 tokens one by one: crosses many pages and attention key blocks."""

@@ -85,6 +85,39 @@ def mixed(requests, seed=0, max_live=4, decode_tail=8):
     return _number(steps)
 
 
+def random_trace(requests, rng, max_live):
+    """Steps drawn at random: requests enter while others run, portions from a few tokens to
+    hundreds beside single tokens, requests that sit a step out, tails of 0 to 40 tokens decoded one
+    by one, logits wanted at some places only."""
+    waiting = list(requests.items())
+    live: dict[str, int] = {}
+    steps = []
+    sizes = rng.choice([(2, 3, 5, 9, 17, 30), (1, 2, 64, 128, 257), (2, 40, 300, 600), (16, 32, 48, 512)])
+    tail = {rid: rng.choice((0, 1, 4, 12, 40)) for rid in requests}
+    while waiting or live:
+        while waiting and len(live) < max_live and (not live or rng.random() < 0.7):
+            rid, _ = waiting.pop(0)
+            live[rid] = 0
+        entries, ended = [], []
+        for rid in list(live):
+            toks = requests[rid]
+            p = live[rid]
+            left = len(toks) - p
+            if rng.random() < 0.2 and entries:
+                continue
+            n = 1 if left <= tail[rid] else min(left - tail[rid], rng.choice(sizes))
+            want = [i for i in range(n) if n <= 4 or rng.random() < 0.3 or i == n - 1]
+            entries.append({"id": rid, "tokens": toks[p: p + n], "want": want})
+            live[rid] = p + n
+            if p + n == len(toks):
+                ended.append(rid)
+        for rid in ended:
+            del live[rid]
+        if entries:
+            steps.append({"entries": entries, "end": ended})
+    return _number(steps)
+
+
 def _number(steps):
     for i, s in enumerate(steps):
         s["step"] = i
