@@ -663,7 +663,9 @@ class HipOps:
         self._launch_attention(q, out, cache, ctx, nq, nkv, d, scale, window, None, False)
 
     def _launch_attention(self, q, out, cache, ctx, nq, nkv, d, scale, window, subset, decode, own=None):
-        """One launch over the sequences in ``subset`` (None: all of the step's)."""
+        """One launch over the sequences in ``subset`` (None: all of the step's). ``own``: the
+        decode kernel takes the tokens' queries, own keys and own values from the q/k/v product
+        (``decode_attention``); ``q`` is then None."""
         lib = attention_library(d)
         g = nq // nkv
         if subset is None:  # the step's own maxima: under a graph they are those of its bucket
