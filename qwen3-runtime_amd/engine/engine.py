@@ -97,6 +97,15 @@ class Engine:
             self._broken = f"{type(exc).__name__}: {exc}"
             raise
 
+    def _next_step_is_known(self, batch: list[Request], to_sample: list[Request]) -> bool:
+        """Whatever ids this step's sampling gives, the next step is the same requests with one
+        token each: all of them decode, none can end with the next token (stop ids do not count
+        for it and its limit is further off), and nobody else holds pages or waits."""
+        if len(to_sample) != len(batch) or self.scheduler.queue or len(self.scheduler.residents) != len(batch):
+            return False
+        return all(r.grant == 1 and not r.stop.stop_ids_count and r.num_output_tokens + 1 < r.stop.limit
+                   for r in batch)
+
     def _run_step(self, batch: list[Request], evictions_before: int):
         entries, to_sample = [], []
         n_prompt = n_decode = 0
@@ -121,7 +130,11 @@ class Engine:
             slot_rows = self.runner.last_row_slots
             if logits is None or slot_rows is None or slot_rows.numel() != len(to_sample):
                 raise RuntimeError("the step's logits do not match the requests to sample for")
-            ids, logprobs = self.sampler.sample(logits, slot_rows, to_sample)
+            drawn = self.sampler.launch(logits, slot_rows, to_sample)
+            if self._next_step_is_known(batch, to_sample):
+                # the device goes on with the next step while the host waits for this one's ids
+                self.runner.step_ahead(drawn.tokens)
+            ids, logprobs = self.sampler.finish(drawn)
             for req, tok, lp in zip(to_sample, ids, logprobs):
                 new_token[req.request_id] = tok
                 req.logprobs.append(lp)

@@ -53,6 +53,8 @@ class DecodeGraph:
         self._last_epoch = -1  # the cache's epoch at the last fill: a later one voids the buffer
         self._host_views = None
         self._row_index = None
+        self._prepared = False  # the host buffer holds the step after the one launched last
+        self._ahead = None      # (requests, lengths, epoch) of a step launched before it was asked for
 
     def _fill(self, entries: Sequence[StepEntry]):
         runner = self.runner
@@ -154,12 +156,42 @@ class DecodeGraph:
         except CacheFull:
             return
         self._advance(rids, starts)
+        self._prepared = True
+
+    def launch_ahead(self, tokens: torch.Tensor) -> bool:
+        """Launch the step that ``prepare_next`` has prepared, now, with the ids that the sampler
+        has just written on the device (int32 [batch], in the step's order), before the host has
+        seen them. The caller knows that the step will be asked for: no request ends with these
+        ids, and nobody else waits. ``run`` then finds its work done. If something else is asked
+        for instead (a request added or cancelled in between), the launch has only written keys
+        and values at positions that the cache's books do not count, into pages reserved for
+        them; whoever owns such a page later writes a position before reading it."""
+        if not self._prepared or self.graph is None or tokens.shape != (self.batch,):
+            return False
+        self._prepared = False
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+        self.views_dev["ids"].copy_(tokens)
+        self.runner.last_row_slots = self.views_dev["row_slots"]
+        self.graph.replay()
+        self._ahead = (list(self._last_rids), list(self._last_starts), self._last_epoch, self.runner.steps_begun)
+        return True
 
     def _views(self):
         return {name: self.dev[off: off + int(np.prod(shape))].view(shape) for name, off, shape in self.layout}
 
     def run(self, entries: Sequence[StepEntry]):
         runner = self.runner
+        ahead, self._ahead = self._ahead, None
+        self._prepared = False
+        if ahead is not None:
+            rids = [e.request_id for e in entries]
+            # the very next step of the runner (no other has used the graphs' shared memory since),
+            # for the same requests at the same lengths, owning the same pages
+            if ahead == (rids, [runner.cache.length(r) for r in rids], runner.cache.epoch, runner.steps_begun - 1):
+                runner.last_row_slots = self.views_dev["row_slots"]
+                runner.steps_ahead[1] += 1
+                return self.logits  # launched already, with the ids these entries bring
         packed = self._fill(entries)
         if self.graph is None:
             if self.ctx is None:

@@ -44,9 +44,18 @@ class ModelRunner:
         self._pinned: torch.Tensor | None = None
         self._copied = torch.cuda.Event() if self.device.type == "cuda" else None
         self.graph_max_batch = 256
+        self.steps_begun = 0
+        self._last_graph = None
+        # A step may be launched before it is asked for, and then not be asked for after all, only
+        # if running it has no effect that a later step could see: keys and values written beyond
+        # a request's counted length are such; a per-request state that the step replaces is not.
+        self.repeatable = all(s.kind == "paged_kv" for s in model.plan.caches)
+        self.steps_ahead = [0, 0]  # launched before they were asked for; of these, asked for
 
     # ---- public ------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
+        self.steps_begun += 1
+        self._last_graph = None
         for e in entries:
             end = self.cache.length(e.request_id) + len(e.tokens)
             if end > self.max_model_len:
@@ -68,7 +77,19 @@ class ModelRunner:
             self.cache.commit(e.request_id, len(e.tokens))
         if graph is not None:
             graph.prepare_next()  # host work for the next step while the GPU runs this one
+        self._last_graph = graph
         return logits
+
+    def step_ahead(self, tokens: torch.Tensor) -> bool:
+        """The step just run was a replayed decode step, and the caller knows that the next one
+        will be the same requests, each with the id that ``tokens`` (int32, on the device, in the
+        step's order) holds for it: launch that step now. The next ``step`` must still be called,
+        with those ids; it finds its logits computed. Returns whether anything was launched."""
+        graph = self._last_graph
+        if not self.repeatable or graph is None or not graph.launch_ahead(tokens):
+            return False
+        self.steps_ahead[0] += 1
+        return True
 
     # ---- eager path ----------------------------------------------------------
     def _upload(self, packed: PackedStep) -> dict[str, torch.Tensor]:

@@ -29,6 +29,9 @@ class Sampler:
         self.iparams = slots.add_tensor("sampler_i32", (2,), torch.int32, survives_restart=True)
         self.seeds = slots.add_tensor("sampler_seed", (2,), torch.int64, survives_restart=True)
         self.counts: torch.Tensor | None = None
+        # where sampled ids land on the host: pinned, so that the copy does not wait for the host
+        self._landing: torch.Tensor | None = None
+        self._landed = torch.cuda.Event() if self.device.type == "cuda" else None
 
     def admit(self, slot: int, params: SamplingParams, seed: int, prompt: Sequence[int]) -> None:
         """Write the request's options into its slot (zeroed when the slot was taken)."""
@@ -47,6 +50,12 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, slot_rows: torch.Tensor, reqs) -> tuple[list[int], list[float]]:
         """``logits`` [R, V] float32; ``slot_rows`` int32 [R]; ``reqs`` the R requests in row order."""
+        return self.finish(self.launch(logits, slot_rows, reqs))
+
+    def launch(self, logits: torch.Tensor, slot_rows: torch.Tensor, reqs) -> "Drawn":
+        """Everything of ``sample`` that the host does not wait for: the kernels, and the copy of
+        ids and log-probabilities to host memory. ``Drawn.tokens`` stays on the device, for a
+        caller that feeds the next step from there."""
         bias = [(i, t, v) for i, r in enumerate(reqs) for t, v in (r.sampling.logit_bias or {}).items()]
         if bias:
             logits = logits.clone()
@@ -68,5 +77,28 @@ class Sampler:
                     lp[i] = logp[i, int(f)]
         if self.counts is not None:
             self.ops.count_tokens(self.counts, slot_rows, tok)
-        host = both.cpu()  # ids and log-probabilities in one copy, one wait
+        if both.device.type != "cuda":
+            return Drawn(tok, both, None)
+        n = both.numel()
+        if self._landing is None or self._landing.numel() < n:
+            self._landing = torch.empty(max(n, 512), dtype=torch.int32, pin_memory=True)
+        host = self._landing[:n].view(both.shape)
+        host.copy_(both, non_blocking=True)  # ids and log-probabilities in one copy
+        self._landed.record()
+        return Drawn(tok, host, self._landed)
+
+    def finish(self, drawn: "Drawn") -> tuple[list[int], list[float]]:
+        """Wait for what ``launch`` started (one wait); one ``launch`` is open at a time."""
+        if drawn.landed is not None:
+            drawn.landed.synchronize()
+        host = drawn.host if drawn.landed is not None else drawn.host.cpu()
         return host[0].tolist(), host[1].view(torch.float32).tolist()
+
+
+class Drawn:
+    """A ``Sampler.launch`` under way: the ids on the device, and where they arrive on the host."""
+
+    __slots__ = ("tokens", "host", "landed")
+
+    def __init__(self, tokens, host, landed):
+        self.tokens, self.host, self.landed = tokens, host, landed

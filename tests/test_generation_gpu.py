@@ -61,6 +61,46 @@ def test_graph_replay_equals_eager(model_folders, dtype):
     assert m.generate(prompts, max_tokens=40) == eager
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_launched_before_they_are_asked_for(model_folders, dtype):
+    """While the host waits for a decode step's ids the device already runs the next step, if
+    nothing can make that step another one. The tokens are those of an engine that never does
+    so, also where a launched step is not asked for after all: a request arrives, one is
+    cancelled, one may stop at an id, a limit is reached."""
+    from qwen3_runtime_amd.sampling.params import SamplingParams
+
+    cfg, _ = P.read_model(model_folders["tiny_b"])
+    prompts = prompts_for(cfg, [30, 9, 61, 5], seed=8)
+    params = [SamplingParams(temperature=0.7, seed=40 + i, repetition_penalty=1.2 if i == 1 else 1.0)
+              for i in range(4)]
+
+    def run(ahead: bool):
+        eng = llm(model_folders["tiny_b"], dtype=dtype, graph=True, pages=128).engine
+        eng.runner.repeatable = ahead
+        reqs = [eng.request(eng.add_request(prompts[i], 60 - 7 * i, sampling=params[i])) for i in range(2)]
+        for _ in range(20):
+            eng.step()
+        reqs.append(eng.request(eng.add_request(prompts[2], 30, sampling=params[2])))  # arrives in between
+        for _ in range(15):
+            eng.step()
+        eng.finish_request(reqs[1].request_id)                                        # cancelled in between
+        for _ in range(5):
+            eng.step()
+        late = eng.add_request(prompts[3], 25, sampling=params[3], ignore_eos=False, stop_token_ids=(3,))
+        reqs.append(eng.request(late))
+        while not eng.is_finished():
+            eng.step()
+        eng.cache.check()
+        assert eng.cache.num_free_pages == 128
+        return [(r.output_tokens, r.finish_reason) for r in reqs], eng.runner.steps_ahead
+
+    plain_order, none = run(False)
+    assert none == [0, 0]
+    ahead_order, (launched, taken) = run(True)
+    assert ahead_order == plain_order
+    assert taken >= 20 and launched > taken, (launched, taken)  # most were asked for, some were not
+
+
 def test_the_collector_stays_out_of_a_capture(model_folders):
     """An engine with captured graphs, dropped while part of a reference cycle, lives on until the
     collector of cycles runs. If that happened inside a later engine's capture, the old graphs
