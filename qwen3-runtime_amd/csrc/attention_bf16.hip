@@ -253,21 +253,24 @@ __device__ __forceinline__ void block_pages(const int* __restrict__ table, int b
 // ONCE: the block is the only reader of these keys and values in the step (decoding: one block
 // per sequence and key head serves the whole group of query heads), so they are loaded
 // non-temporally and leave the caches alone.
+// live = false (uniform over the wave): a load past the wave's last block, issued only so that
+// the loop has one shape; every lane then reads the cache's first bytes, a few lines for the
+// whole wave, instead of a block of keys and values that nobody uses.
 template <bool P2, bool ONCE = false>
 __device__ __forceinline__ void block_load(const AttnTileArgs& a, int kvh, int base, int lo, int pos_max, int r16,
-                                           int quad, const int pg[3], KvBlock& blk) {
+                                           int quad, const int pg[3], KvBlock& blk, bool live = true) {
   const int ps = a.page_size;
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
     const int kidx = min(max(base + 8 * (r16 >> 2) + 4 * kb + (r16 & 3), lo), pos_max);
-    const bf16_t* kp = a.k_cache + (((size_t)pg[kb] * a.nkv + kvh) * ps + page_mod<P2>(kidx, ps)) * D;
+    const bf16_t* kp = live ? a.k_cache + (((size_t)pg[kb] * a.nkv + kvh) * ps + page_mod<P2>(kidx, ps)) * D : a.k_cache;
 #pragma unroll
     for (int i = 0; i < KFULL; ++i)
       blk.k[kb][i] = ONCE ? load_once8(kp + 32 * i + 8 * quad) : *(const bf16x8_t*)(kp + 32 * i + 8 * quad);
     if (KTAIL) blk.kt[kb] = load_tail(kp + 32 * KFULL, quad);
   }
   const int kv0 = min(max(base + 8 * quad, lo & ~7), pos_max & ~7);
-  const bf16_t* vp = a.v_cache + (((size_t)pg[2] * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps);
+  const bf16_t* vp = live ? a.v_cache + (((size_t)pg[2] * a.nkv + kvh) * D + r16) * ps + page_mod<P2>(kv0, ps) : a.v_cache;
 #pragma unroll
   for (int i = 0; i < DB; ++i)
     blk.v[i] = ONCE ? load_once8(vp + (size_t)16 * i * ps) : *(const bf16x8_t*)(vp + (size_t)16 * i * ps);
@@ -862,24 +865,28 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
       if (KTAIL) qtail = load_tail(qp + 32 * KFULL, quad);
     }
 
-    // keys and values are loaded one block ahead, page numbers two; past the wave's last block
-    // the loads repeat that block (their data is not used)
+    // two blocks of keys and values are on their way while a third is multiplied, and the page
+    // numbers of the two after them; past the wave's last block the loads go on (one shape of
+    // loop, no load under a branch) but fetch next to nothing
     const int last = b + (b1 - 1 - b) / DW * DW;
     KvBlock A, B;
     int pgA[3], pgB[3];
     block_pages<P2>(table, b << 5, lo, pos_max, a.page_size, r16, quad, pgA);
     block_pages<P2>(table, min(b + DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
     block_load<P2, DECODE_ONCE>(a, kvh, b << 5, lo, pos_max, r16, quad, pgA, A);
+    block_load<P2, DECODE_ONCE>(a, kvh, min(b + DW, last) << 5, lo, pos_max, r16, quad, pgB, B, b + DW <= last);
+    block_pages<P2>(table, min(b + 2 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
+    block_pages<P2>(table, min(b + 3 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
     if (FUSED) own_token();  // while the first keys and values are on their way
     while (true) {
-      block_load<P2, DECODE_ONCE>(a, kvh, min(b + DW, last) << 5, lo, pos_max, r16, quad, pgB, B);
-      block_pages<P2>(table, min(b + 2 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
       block_compute(A, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.scale_log2, m, l, o);
+      block_load<P2, DECODE_ONCE>(a, kvh, min(b + 2 * DW, last) << 5, lo, pos_max, r16, quad, pgA, A, b + 2 * DW <= last);
+      block_pages<P2>(table, min(b + 4 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgA);
       b += DW;
       if (b >= b1) break;
-      block_load<P2, DECODE_ONCE>(a, kvh, min(b + DW, last) << 5, lo, pos_max, r16, quad, pgA, A);
-      block_pages<P2>(table, min(b + 2 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
       block_compute(B, qreg, qtail, b << 5, lo, pos_min, pos_max, quad, row_valid, qpos_c, window, a.scale_log2, m, l, o);
+      block_load<P2, DECODE_ONCE>(a, kvh, min(b + 2 * DW, last) << 5, lo, pos_max, r16, quad, pgB, B, b + 2 * DW <= last);
+      block_pages<P2>(table, min(b + 4 * DW, last) << 5, lo, pos_max, a.page_size, r16, quad, pgB);
       b += DW;
       if (b >= b1) break;
     }
