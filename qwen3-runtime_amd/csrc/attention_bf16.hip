@@ -650,6 +650,41 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   }
 }
 
+// Few splits: every load is asked for before the first is used (clamped indices, so none stands
+// under a branch), one trip to memory instead of two; the sums are those of the kernel's loop.
+// A thread takes elements threadIdx.x and threadIdx.x + blockDim.x of the row.
+template <int MAX>
+__device__ __forceinline__ void merge_few(const float* __restrict__ part_o, const float* __restrict__ lse,
+                                          bf16_t* __restrict__ out, int num_splits, size_t row) {
+  float ls[MAX], pv[2][MAX];
+  const int d0 = min((int)threadIdx.x, D - 1), d1 = min((int)(threadIdx.x + blockDim.x), D - 1);
+#pragma unroll
+  for (int s = 0; s < MAX; ++s) {
+    const int sc = min(s, num_splits - 1);
+    ls[s] = lse[sc];
+    pv[0][s] = part_o[(row * num_splits + sc) * D + d0];
+    pv[1][s] = part_o[(row * num_splits + sc) * D + d1];
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < MAX; ++s) mx = fmaxf(mx, ls[s]);
+  float acc[2] = {0.f, 0.f}, wsum = 0.f;
+  if (mx != -INFINITY) {
+#pragma unroll
+    for (int s = 0; s < MAX; ++s) {
+      if (s < num_splits) {
+        const float w = exp2f(ls[s] - mx);
+        wsum += w;
+        acc[0] += w * pv[0][s];
+        acc[1] += w * pv[1][s];
+      }
+    }
+  }
+  if ((int)threadIdx.x < D) out[row * D + threadIdx.x] = (bf16_t)(wsum > 0.f ? acc[0] / wsum : 0.f);
+  if ((int)(threadIdx.x + blockDim.x) < D)
+    out[row * D + threadIdx.x + blockDim.x] = (bf16_t)(wsum > 0.f ? acc[1] / wsum : 0.f);
+}
+
 // out[row] = sum_s 2^(lse_s - M) O_s / sum_s 2^(lse_s - M); empty splits weigh 0
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse,
                                        bf16_t* __restrict__ out, int num_splits, const int* __restrict__ tokens,
@@ -657,6 +692,11 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
   // rows are (token, query head); with a token list the grid walks the listed tokens' rows only
   const size_t row = tokens ? (size_t)tokens[blockIdx.x / nq] * nq + blockIdx.x % nq : blockIdx.x;
   const float* lse = part_lse + row * num_splits;
+  if (num_splits <= 16 && D <= 2 * (int)blockDim.x) {
+    if (num_splits <= 8) merge_few<8>(part_o, lse, out, num_splits, row);
+    else merge_few<16>(part_o, lse, out, num_splits, row);
+    return;
+  }
   float mx = -INFINITY;
   for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, lse[s]);
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
