@@ -168,6 +168,26 @@ class CacheManager:
                 table.append(g.pool.take(rid))
         self._reserved[rid] = max(self._reserved[rid], end)
 
+    def trim(self) -> int:
+        """Give back every page that a request holds only for tokens it has reserved and not
+        stored (pages taken ahead for a step that then was not the next one). Returns how many
+        went back; tables that were handed out before are void then, as after any loss of pages."""
+        returned = 0
+        for rid, length in self._length.items():
+            if self._reserved[rid] <= length:
+                continue
+            for g in self.groups:
+                table = g.tables[rid]
+                while len(table) > g.pages_for(length):
+                    page = table.pop()
+                    if page >= 0:
+                        g.pool.give(page, rid)
+                        returned += 1
+            self._reserved[rid] = length
+        if returned:
+            self.epoch += 1
+        return returned
+
     def commit(self, rid: Hashable, num_tokens: int) -> None:
         """``num_tokens`` more tokens are stored. Window groups give back what no query sees."""
         new_len = self._length[rid] + num_tokens

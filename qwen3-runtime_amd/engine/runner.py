@@ -21,6 +21,7 @@ from typing import Sequence
 import numpy as np
 import torch
 
+from ..cache.pages import CacheFull
 from ..parts.base import GroupView, StepContext
 from .batch import PackedStep, StepEntry, pack_step
 
@@ -62,8 +63,16 @@ class ModelRunner:
                 raise ValueError(
                     f"request {e.request_id!r} would reach {end} tokens; the limit is {self.max_model_len}"
                 )
-        for e in entries:
-            self.cache.reserve(e.request_id, len(e.tokens))
+        try:
+            for e in entries:
+                self.cache.reserve(e.request_id, len(e.tokens))
+        except CacheFull:
+            # A replayed decode step takes the pages of the step it expects next while the device
+            # runs; if another step comes instead and finds no page, those go back first.
+            if not self.cache.trim():
+                raise
+            for e in entries:
+                self.cache.reserve(e.request_id, len(e.tokens))
         pure_decode = all(len(e.tokens) == 1 for e in entries)
         graph = None
         if self.hip_graph and pure_decode and len(entries) <= self.graph_max_batch:

@@ -72,6 +72,34 @@ def test_decoding_takes_a_page_only_when_crossing_one():
     assert len(m.block_table(0, "r")) == 2
 
 
+def test_trim_gives_back_pages_reserved_and_not_stored():
+    """Pages taken ahead for a step that then does not come: back to the pool, stored tokens
+    untouched, and the epoch says that tables handed out before are void."""
+    window = CacheSpec("paged_kv", heads=1, head_dim=8, window=6)
+    m = manager(6, 4, [FULL, window])
+    m.admit("a")
+    m.admit("b")
+    advance(m, "a", 8)          # two pages in the full group; the window group has given one back
+    advance(m, "b", 3)
+    m.reserve("a", 1)           # the page of token 8, ahead of its step
+    m.reserve("b", 6)           # two pages more, ahead
+    held = {rid: [list(m.block_table(g, rid)) for g in range(2)] for rid in "ab"}
+    assert len(held["a"][0]) == 3 and len(held["b"][0]) == 3
+    free_before, epoch = [g.pool.num_free for g in m.groups], m.epoch
+    assert m.trim() == 2 * (1 + 2)
+    m.check()
+    assert [g.pool.num_free for g in m.groups] == [f + 3 for f in free_before] and m.epoch == epoch + 1
+    for rid, n in (("a", 2), ("b", 1)):
+        for g in range(2):
+            assert m.block_table(g, rid) == held[rid][g][:n]
+    assert m.length("a") == 8 and m.length("b") == 3
+    with pytest.raises(AssertionError):
+        m.commit("a", 1)        # the reservation is gone with the pages
+    advance(m, "a", 1)
+    assert m.trim() == 0 and m.epoch == epoch + 1
+    m.check()
+
+
 def test_release_returns_everything_and_freed_pages_come_out_last():
     m = manager(8, 16)
     m.admit("a")
@@ -234,6 +262,15 @@ def test_random_lifetimes_keep_every_page_accounted_for(seed, num_pages, page_si
                 slots = m.token_slots(0, rid, before, n)
                 assert len(set(slots.tolist())) == n
                 m.commit(rid, n)
+        elif op < 0.86 and live:
+            rid = rng.choice(live)      # pages taken ahead, and given back before they are used
+            ahead = m.max_reservable_tokens(rid, rng.choice([1, 9]))
+            m.reserve(rid, ahead)
+            if rng.random() < 0.5:
+                lengths = {r: m.length(r) for r in live}
+                m.trim()
+                assert {r: m.length(r) for r in live} == lengths
+                assert all(len(m.block_table(0, r)) == m.groups[0].pages_for(m.length(r)) for r in live)
         elif op < 0.9 and live:
             m.restart(rng.choice(live))
         elif live:

@@ -531,6 +531,45 @@ def test_graph_buffer_is_repacked_when_a_request_id_comes_back(model_folders):
     torch.testing.assert_close(replayed, torch.cat([want[30:34], want[34:38]]).float(), atol=5e-5, rtol=5e-5)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_taken_ahead_by_a_replayed_step_go_back_when_another_step_needs_them(model_folders, dtype):
+    """While the device runs a replayed decode step, the host takes the pages of the step it
+    expects next. With a pool that holds exactly the live tokens, a different next step (another
+    request's prompt) finds no page; the pages taken ahead then go back and the step runs."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.batch import StepEntry
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg, _ = P.read_model(model_folders["tiny_b"])
+    ids, other = prompts_for(cfg, [24, 8], seed=21)
+
+    def run(graph):
+        loaded = load(model_folders["tiny_b"], EngineConfig(page_size=8, num_pages=3, max_num_seqs=2, dtype=dtype,
+                                                            device=DEV, hip_graph=graph))
+        runner, cache = loaded.runner, loaded.cache
+        out = []
+        cache.admit("a")
+        runner.step([StepEntry("a", ids[:13], [])])
+        for p in range(13, 16):                       # eager, capture, replay: "a" now fills two pages
+            out.append(runner.step([StepEntry("a", ids[p: p + 1], [0])])[0].cpu().clone())
+        ahead = cache.num_free_pages == 0             # the third page was taken for token 16
+        cache.admit("b")
+        out.append(runner.step([StepEntry("b", other[:8], [7])])[0].cpu().clone())  # needs that page
+        cache.release("b")
+        for p in range(16, 19):
+            out.append(runner.step([StepEntry("a", ids[p: p + 1], [0])])[0].cpu().clone())
+        cache.check()
+        return torch.stack(out), ahead
+
+    eager, _ = run(False)
+    replayed, ahead = run(True)
+    assert ahead, "the replayed step did not take its next page ahead: the case is not met"
+    if dtype == "float32":
+        torch.testing.assert_close(replayed, eager, atol=2e-5, rtol=2e-5)
+    else:  # other key splits under the graph: rounding noise, in units of the logits' spread
+        assert float((replayed - eager).pow(2).mean().sqrt() / eager.std()) < 0.015
+
+
 def test_sampler_with_an_excluded_id():
     """A bias of -inf excludes an id: the row's first value being -inf must not poison the sum
     of exponentials (greedy log-probability) nor be drawn."""
