@@ -421,6 +421,59 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
 // the LDS serves lanes 0-7 together with lanes 24-31, and so on, 64 banks of 4 bytes. The
 // kernel's time did not change with it: it is not bound by LDS reads.)
 constexpr int KROW = D % 32 == 0 ? D + 16 : D;  // elements per key row in LDS
+// Two tiles of a wave meet a block of 32 keys, with the rows' reference maxima moved lazily.
+// The exponentials are taken against a reference m that may lie below the row's true maximum by
+// up to LAZY (in units of the scaled scores, base 2): probabilities then reach 2^LAZY at most,
+// which bfloat16 and the float32 sums hold as well as values below one, and the quotient of
+// accumulator and sum does not change. As long as no score of the wave rises above its row's
+// reference by more than that, and no tile touches the diagonal or a window's edge, a round is
+// two stretches of code without a branch: products and lane-local maxima, then exponentials and
+// second products, which the compiler can place side by side. No maximum across the four lanes
+// of a row, no factor for the accumulator, no test whether it moved. Otherwise (the first block
+// of keys, the blocks at the diagonal, a row whose scores jump) the reference is set to the true
+// maximum and the accumulator shrunk as in tiles_update.
+constexpr float LAZY = 8.0f;
+
+__device__ __forceinline__ void tile_mask(f32x4_t sc[2], int base, int quad, bool row_valid, int qpos, int window) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int key = base + 8 * quad + e;
+    const bool vis = row_valid && key <= qpos && (window == 0 || key > qpos - window);
+    sc[e >> 2][e & 3] = vis ? sc[e >> 2][e & 3] : -INFINITY;
+  }
+}
+
+__device__ __forceinline__ float lane_max(const f32x4_t sc[2]) {
+  float mx = -INFINITY;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) mx = max2(mx, sc[e >> 2][e & 3]);
+  return mx;
+}
+
+// the slow part: reference to the true maximum, sum and accumulator shrunk to it
+__device__ __forceinline__ void tile_move_reference(float lane_mx, float scale_log2, float& m, float& l, f32x4_t* o) {
+  const float m_new = max2(m, row_max4(lane_mx) * scale_log2);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
+  const float corr = __builtin_amdgcn_exp2f(m - m_use);
+  m = m_new;
+  l *= corr;
+#pragma unroll
+  for (int i = 0; i < DB; ++i) o[i] *= corr;
+}
+
+__device__ __forceinline__ void tile_probabilities(const f32x4_t sc[2], float scale_log2, float m, float& l,
+                                                   bf16x8_t& pb) {
+  const float m_use = m == -INFINITY ? 0.f : m;
+  float psum = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float pe = __builtin_amdgcn_exp2f(fmaf(sc[e >> 2][e & 3], scale_log2, -m_use));
+    psum += pe;
+    pb[e] = (bf16_t)pe;
+  }
+  l += psum;
+}
+
 constexpr int VROW = 48;                        // elements per value row (one head element, 32 keys) in LDS
 constexpr int STAGE_ELEMS = 32 * KROW + D * VROW;
 
@@ -479,7 +532,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
     const int row_last = min(row0 + 16 * RT - 1, n_rows - 1);
     const int pos_min = first_pos + row0 / g, pos_max = first_pos + row_last / g;
     wb0 = (a.window > 0 ? max(0, pos_min - a.window + 1) : 0) >> 5;
-    wb1 = (pos_max >> 5) + 1;
+    wb1 = min((pos_max >> 5) + 1, b1);  // not into the next split's blocks
   }
 
   f32x4_t o[RT][DB];
@@ -579,10 +632,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
 #pragma unroll
       for (int i = 0; i < DB; ++i) vv[i] = *(const bf16x8_t*)(vb + (16 * i + r16) * VROW + 8 * quad);
 
-      f32x4_t sc[RT][2];
-      unsigned whole = 0;
-#pragma unroll
-      for (int t = 0; t < RT; ++t) {
+      auto scores = [&](int t, f32x4_t sc[2]) {
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -590,13 +640,49 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
           for (int i = 0; i < KFULL; ++i)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk[s2][i], qreg[t][i], acc, 0, 0, 0);
           if (KTAIL) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[s2], qtail[t], acc, 0, 0, 0);
-          sc[t][s2] = acc;
+          sc[s2] = acc;
         }
-        // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
-        const int sees_all = (base + 31 <= tile_pos_min[t]) & ((a.window == 0) | (base > tile_pos_max[t] - a.window));
-        whole |= (unsigned)sees_all << t;
+      };
+      // every row of the tile sees the whole block unless it touches the diagonal or the window's edge
+      auto sees_all = [&](int t) {
+        return (base + 31 <= tile_pos_min[t]) & ((a.window == 0) | (base > tile_pos_max[t] - a.window));
+      };
+      if constexpr (RT == 2) {
+        f32x4_t sc0[2], sc1[2];
+        bf16x8_t pb0, pb1;
+        scores(0, sc0);
+        scores(1, sc1);
+        const bool edge = !(sees_all(0) & sees_all(1));  // the same for the whole wave
+        float mx0 = lane_max(sc0), mx1 = lane_max(sc1);
+        const bool jumps = mx0 * a.scale_log2 > m[0] + LAZY || mx1 * a.scale_log2 > m[1] + LAZY;
+        if (edge || __any(jumps)) {
+          if (!sees_all(0)) {
+            tile_mask(sc0, base, quad, row_valid[0], qpos[0], a.window);
+            mx0 = lane_max(sc0);
+          }
+          if (!sees_all(1)) {
+            tile_mask(sc1, base, quad, row_valid[1], qpos[1], a.window);
+            mx1 = lane_max(sc1);
+          }
+          tile_move_reference(mx0, a.scale_log2, m[0], l[0], o[0]);
+          tile_move_reference(mx1, a.scale_log2, m[1], l[1], o[1]);
+        }
+        tile_probabilities(sc0, a.scale_log2, m[0], l[0], pb0);
+        tile_probabilities(sc1, a.scale_log2, m[1], l[1], pb1);
+#pragma unroll
+        for (int i = 0; i < DB; ++i) o[0][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[i], pb0, o[0][i], 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < DB; ++i) o[1][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[i], pb1, o[1][i], 0, 0, 0);
+      } else {
+        f32x4_t sc[RT][2];
+        unsigned whole = 0;
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+          scores(t, sc[t]);
+          whole |= (unsigned)sees_all(t) << t;
+        }
+        tiles_update<RT>(sc, vv, whole, base, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
       }
-      tiles_update<RT>(sc, vv, whole, base, quad, row_valid, qpos, a.window, a.scale_log2, m, l, o);
     }
   };
   int page = lookup(b_first);
@@ -611,14 +697,17 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
     fetch(min(b + 2, b_last), page, set_a);
     page = lookup(min(b + 3, b_last));
     multiply(b, 0);
-    if (b + 1 < b1) stash(b + 1, 1, set_b);
+    stash(min(b + 1, b_last), 1, set_b);
     __syncthreads();
-    if (b + 1 >= b1) break;
-    // odd round: set B is free, set A holds block b + 2
+    // odd round: set B is free, set A holds block b + 2. With an odd number of blocks the last
+    // odd round has nothing to multiply (b + 1 == b1 lies outside every wave's range) and only
+    // fetches and stores the last block once more. Leaving the loop here instead gave the
+    // compiler a path back to the loop's head with set A's loads in flight, and made it wait
+    // for every load at the head of every round.
     fetch(min(b + 3, b_last), page, set_b);
     page = lookup(min(b + 4, b_last));
     multiply(b + 1, 1);
-    if (b + 2 < b1) stash(b + 2, 0, set_a);
+    stash(min(b + 2, b_last), 0, set_a);
     __syncthreads();
   }
 

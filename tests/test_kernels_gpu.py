@@ -640,6 +640,33 @@ def test_attention_far_key_stands_out(ops):
         close(got, want, 1e-2, 1e-2)
 
 
+@pytest.mark.parametrize("rise,jump_at", [(0.0, None), (5.0, None), (7.5, None), (3.0, 9), (0.5, 0)])
+def test_prompt_attention_with_scores_that_climb(ops, rise, jump_at):
+    """The prompt kernel takes its exponentials against a reference that follows a row's maximum
+    only when a score rises above it by more than 2^8. Keys are made so that every block of 32
+    lifts the maximum by ``rise`` (base-2 units of the scaled score: below the threshold, the
+    reference stays behind and probabilities above one are summed), and one block by 30 (the
+    reference must move and what was summed before must shrink). Values differ block by block,
+    so a block weighed wrongly shows."""
+    nq, nkv, d, ps, n = 8, 2, 128, 16, 640
+    q, cache, ctx = build_attention_case([(n, n)], nq, nkv, d, ps, torch.bfloat16, seed=5, shuffle=True)
+    table = cache.group.block_table[0].cpu()
+    q[:] = 0
+    q[:, ::d] = 1.0                                    # every head looks at element 0 of the keys
+    ln2 = math.log(2.0)
+    for pos in range(n):
+        block = pos // 32
+        level = rise * block + (30.0 if jump_at is not None and block >= jump_at else 0.0)
+        page, off = int(table[pos // ps]), pos % ps
+        cache.k[page, :, off, :] = 0
+        cache.k[page, :, off, 0] = level * ln2 + 0.01 * (pos % 32)   # score = level (base 2), nearly flat inside a block
+        cache.v[page, :, :, off] = float(block % 7) - 3.0 + 0.125 * (pos % 4)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, 1.0)
+    got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 1.0, None)
+    close(got, want, 2e-2, 2e-2)
+
+
 def test_argmax_first_maximum(ops):
     x = torch.tensor([[1.0, 3.0, 3.0, 2.0], [0.0, 0.0, 0.0, 0.0], [3.0, -1.0, 2.5, 3.0]], device=DEV)
     assert ops.argmax(x).tolist() == [1, 0, 0]
