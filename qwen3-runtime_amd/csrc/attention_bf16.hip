@@ -807,13 +807,15 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
 // Tiles of at most 16 rows (a decoded token's g query heads, or a very short
 // portion): one block of DW waves per (tile, key head, split). The waves take the
 // block's 32-key blocks round-robin, each with its own running maximum, sum and
-// accumulator; the next block's keys and values are loaded while the current one
-// is multiplied, and page numbers are fetched one block further ahead, so that no
-// load waits for another. The waves' results meet in LDS. With several splits each
+// accumulator; the keys and values of the next two blocks are on their way while
+// one is multiplied, and page numbers are fetched two blocks further ahead, so that
+// no load waits for another. The waves' results meet in LDS. With several splits each
 // block writes its normalised part and the base-2 log of its sum, and a second
 // small kernel merges them. (Merging in the block that arrives last at a counter
 // needs a device-scope fence in every block; with one L2 per XCD that fence costs
-// more than the second launch: measured 355 us against 98 us at 64 sequences.)
+// more than the second launch: measured 355 us against 98 us at 64 sequences. With
+// write-through atomic stores in place of the fence it costs what the second launch
+// costs.)
 constexpr int DW = 4;
 
 __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg, bf16x8_t qtail, int base, int lo,
