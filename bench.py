@@ -4,7 +4,10 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one decode step of the whole engine (schedule, graph replay or
-launches, sampling, copy of the sampled ids). The default run has the layer
+launches, sampling, copy of the sampled ids; the engine launches the next
+step's kernels while the host waits for the ids, so a window of K steps holds the
+device work of K steps, the first of them launched just before the window and the
+one after the last inside it). The default run has the layer
 sizes of the Qwen3-4B configuration with seeded random weights, bfloat16, a
 batch of 8 requests whose prompts are 2,048 uniform-random ids, context limit
 8,192, pages of 16 tokens. W untimed steps, then windows of exactly K timed
