@@ -166,8 +166,10 @@ class DecodeGraph:
         for instead (a request added or cancelled in between), the launch has only written keys
         and values at positions that the cache's books do not count, into pages reserved for
         them; whoever owns such a page later writes a position before reading it."""
-        if not self._prepared or self.graph is None or tokens.shape != (self.batch,):
+        if not self._prepared or self.graph is None:
             return False
+        if tokens.shape != (self.batch,) or tokens.dtype != torch.int32 or tokens.device != self.dev.device:
+            raise ValueError(f"ids for the step ahead: int32 [{self.batch}] on {self.dev.device} expected")
         self._prepared = False
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
