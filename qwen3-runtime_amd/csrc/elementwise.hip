@@ -295,6 +295,10 @@ struct QkArgs {
   void* v_cache;
   int num_tokens, nq, nkv, nv, head_dim, page_size;
   float eps;
+  // [T, head_dim] or null: the cosines of the tokens' head_dim / 2 angles, then their sines, as
+  // rope_table makes them. The kernel for many tokens looks them up instead of computing them in
+  // every layer (inv_freq and positions are still given: the kernel for few tokens computes).
+  const float* rope;
 };
 
 template <typename T>
@@ -423,7 +427,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_wide_kernel(QkArgs a, 
     const int t = (int)(item / groups), grp = (int)(item - (long)t * groups);
     const int c = lane & (lph - 1), hl = lane / lph;
     float sn[8], cs[8];
-    if (a.inv_freq) {
+    if (a.rope) {
+      const float* angles = a.rope + (size_t)t * D + 8 * c;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        cs[e] = angles[e];
+        sn[e] = angles[half + e];
+      }
+    } else if (a.inv_freq) {
       const float pos = (float)a.positions[t];
 #pragma unroll
       for (int e = 0; e < 8; ++e) sincos_angle(pos * a.inv_freq[8 * c + e], &sn[e], &cs[e]);

@@ -44,7 +44,7 @@ class _QkArgs(Structure):
         ("q_out", c_void_p), ("k_out", c_void_p), ("v_out", c_void_p),
         ("k_cache", c_void_p), ("v_cache", c_void_p),
         ("num_tokens", c_int), ("nq", c_int), ("nkv", c_int), ("nv", c_int),
-        ("head_dim", c_int), ("page_size", c_int), ("eps", c_float),
+        ("head_dim", c_int), ("page_size", c_int), ("eps", c_float), ("rope", c_void_p),
     ]
 
 
@@ -427,7 +427,15 @@ class HipOps:
     def _qk(self, args: _QkArgs, dtype, num_pages=0):
         self._check(self.lib, self.lib.qrt_qk_norm_rope_store(byref(args), _CODE[dtype], c_long(num_pages), _stream()))
 
-    def qk_norm_rope_store(self, qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions, cache):
+    # tokens from which the step's cosines and sines are computed once (rope_table) and looked up by
+    # every layer, instead of being computed in every layer's kernel
+    rope_table_from_tokens = 256
+
+    def qk_norm_rope_store(self, qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions, cache, ctx=None,
+                           angles_key=None):
+        """Per-head RMSNorm of queries and keys, NeoX rotation, and the write of keys and values into
+        the cache, in one pass over ``qkv``; returns the queries. With the step's context given,
+        the angles of a long step come from ``rope_table`` (``angles_key`` as there)."""
         t, width = qkv.shape
         _need(qkv, "qkv", shape=(t, (nq + 2 * nkv) * d))
         for name, w in (("q_norm", q_w), ("k_norm", k_w)):
@@ -444,6 +452,9 @@ class HipOps:
         a.v_in, a.v_stride = qkv.data_ptr() + (nq + nkv) * d * es, width
         a.q_weight, a.k_weight, a.inv_freq = _addr(q_w), _addr(k_w), _addr(inv_freq)
         a.positions = _addr(positions) if inv_freq is not None else None
+        if inv_freq is not None and ctx is not None and t >= self.rope_table_from_tokens and t == ctx.num_tokens \
+                and positions is ctx.positions:
+            a.rope = self.rope_table(ctx, inv_freq, angles_key).data_ptr()
         a.q_out = q.data_ptr()
         a.num_tokens, a.nq, a.nkv, a.nv, a.head_dim, a.eps = t, nq, nkv, nkv, d, eps
         pages = 0

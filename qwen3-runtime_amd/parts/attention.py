@@ -95,7 +95,8 @@ class GroupedQueryAttention(Mixer):
             # norm, rotation and the cache write in one pass over qkv
             q = ops.qk_norm_rope_store(
                 qkv, nq, nkv, d, self.q_norm, self.k_norm, eps, inv_freq, ctx.positions,
-                cache if cache.writes else None,
+                cache if cache.writes else None, ctx=ctx,
+                angles_key=None if self.position is None else self.position.angles_key,
             )
         else:
             # an encoding the fused kernel has no form for: norm, let it rotate, then store

@@ -165,7 +165,8 @@ class TorchOps:
     def linear_for_residual(self, x, w):
         return linear(x, w, False, self.compute)
 
-    def qk_norm_rope_store(self, qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions, cache):
+    def qk_norm_rope_store(self, qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions, cache, ctx=None,
+                           angles_key=None):
         if cache is None:
             return qk_norm_rope_store(qkv, nq, nkv, d, q_w, k_w, eps, inv_freq, positions,
                                       compute=self.compute)

@@ -327,6 +327,35 @@ def test_qk_norm_rope_store(ops, dtype, nq, nkv, d, ps, theta):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("t,nq,nkv,d,ps", [(300, 8, 2, 128, 16), (257, 3, 1, 32, 8), (512, 4, 4, 256, 16)])
+def test_qk_norm_rope_store_with_the_steps_table_of_angles(ops, dtype, t, nq, nkv, d, ps):
+    """A long step computes its cosines and sines once (``rope_table``) and every layer's kernel
+    looks them up: the same bits as the kernel that computes them itself, and the plain formulas."""
+    from types import SimpleNamespace
+
+    pages = (t + ps - 1) // ps + 2
+    qkv = rnd(t, (nq + 2 * nkv) * d, dtype=dtype, seed=3)
+    qw, kw = 1 + 0.1 * rnd(d, seed=5), 1 + 0.1 * rnd(d, seed=6)
+    inv = (1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    pos = (torch.arange(t, dtype=torch.int32) + 4000).to(DEV)
+    slots = torch.randperm(pages * ps)[:t].to(torch.int32).to(DEV)
+    caches = [make_cache(pages, nkv, ps, d, dtype) for _ in range(3)]
+    for c in caches:
+        c.group.slots = slots
+    ctx = SimpleNamespace(per_pass={}, positions=pos, num_tokens=t)
+    looked_up = ops.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, pos, caches[0], ctx=ctx)
+    assert len(ctx.per_pass) == 1, "the step's table of angles was not made"
+    computed = ops.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, pos, caches[1])
+    close(looked_up, computed, 0, 0)
+    close(caches[0].k, caches[1].k, 0, 0)
+    close(caches[0].v, caches[1].v, 0, 0)
+    want = R.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, pos, caches[2].k, caches[2].v, slots, ps)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    close(looked_up, want, tol, tol)
+    close(caches[0].k, caches[2].k, tol, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("t,nq,nkv,d,ps,start", [(40, 6, 2, 32, 8, 16), (37, 4, 2, 64, 16, 8), (33, 4, 2, 16, 8, 3),
                                                  (700, 32, 8, 128, 16, 0), (9, 3, 1, 48, 8, 0)])
 def test_qk_norm_rope_store_neighbouring_slots(ops, dtype, t, nq, nkv, d, ps, start):
