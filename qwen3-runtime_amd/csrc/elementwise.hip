@@ -183,8 +183,8 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
   dim3 grid(num_out_rows), block(256);
   const bool vec4 = hidden % 4 == 0 && (uintptr_t)residual % 16 == 0 && (uintptr_t)weight % 16 == 0 &&
                     (uintptr_t)out % 16 == 0 && (!delta || (uintptr_t)delta % 16 == 0) && plane_stride % 4 == 0;
-  // planes known to the compiler (0: no delta) where the count is a usual one
-  const int pl = !delta ? 0 : (planes == 1 || planes == 2 || planes == 4 || planes == 8) ? planes : -1;
+  // planes known to the compiler (0: no delta) up to eight of them
+  const int pl = !delta ? 0 : planes >= 1 && planes <= 8 ? planes : -1;
 #define GO(TD, TO, VEC, KEEP, PL)                                                                               \
   add_rmsnorm_kernel<TD, TO, VEC, KEEP, PL><<<grid, block, 0, stream>>>(residual, (const TD*)delta, weight,     \
                                                                         rows, (TO*)out, hidden, eps, planes,    \
@@ -195,7 +195,11 @@ extern "C" int qrt_add_rmsnorm(float* residual, const void* delta, int delta_dty
     else if (pl == 0) GO(TD, TO, 4, 4, 0);                                                                      \
     else if (pl == 1) GO(TD, TO, 4, 4, 1);                                                                      \
     else if (pl == 2) GO(TD, TO, 4, 4, 2);                                                                      \
+    else if (pl == 3) GO(TD, TO, 4, 4, 3);                                                                      \
     else if (pl == 4) GO(TD, TO, 4, 4, 4);                                                                      \
+    else if (pl == 5) GO(TD, TO, 4, 4, 5);                                                                      \
+    else if (pl == 6) GO(TD, TO, 4, 4, 6);                                                                      \
+    else if (pl == 7) GO(TD, TO, 4, 4, 7);                                                                      \
     else if (pl == 8) GO(TD, TO, 4, 4, 8);                                                                      \
     else GO(TD, TO, 4, 4, -1);                                                                                  \
   } while (0)

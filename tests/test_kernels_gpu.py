@@ -60,7 +60,7 @@ def test_add_rmsnorm(ops, dtype, t, h, eps):
     close(ops.add_rmsnorm(res.clone(), None, w, eps, dtype), R.add_rmsnorm(res.clone(), None, w, eps, dtype), tol, tol)
 
 
-@pytest.mark.parametrize("planes", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("planes", [1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("t,h", [(3, 2560), (2, 5000), (4, 4096), (5, 101), (1, 8)])
 def test_add_rmsnorm_sums_planes_in_order(ops, planes, t, h):
     """The delta in planes [P, T, H] (float32): the residual becomes ((res + p0) + p1) + ..., bit
