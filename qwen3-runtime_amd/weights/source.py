@@ -132,11 +132,14 @@ def write_model_folder(
     norm_jitter: float = 0.1,
     store_dtype: torch.dtype = torch.bfloat16,
     f32_names: Sequence[str] = (),
+    device: torch.device | str = "cpu",
 ) -> Path:
     """Random-weights mode: write ``config.json`` and ``model.safetensors``.
 
     The architecture named by ``config_json`` decides which tensors exist.
     Names in ``f32_names`` are stored in float32 instead of ``store_dtype``.
+    ``device``: where the values are drawn (a GPU draws a model of a real width in
+    seconds where the host takes minutes; the values of a seed differ between devices).
     """
     from safetensors.torch import save_file
 
@@ -149,10 +152,10 @@ def write_model_folder(
     source = RandomSource(decls, seed, std=std, norm_jitter=norm_jitter, store_dtype=torch.float32)
     tensors = {}
     for decl in decls:
-        t = source.get(decl.file_name)
+        t = source.get(decl.file_name, device)
         keep_f32 = decl.file_name in f32_names or decl.storage == "int"  # integers stay int32
         # round through the storage type so that every reader sees equal values
-        tensors[decl.file_name] = (t if keep_f32 else t.to(store_dtype)).contiguous()
+        tensors[decl.file_name] = (t if keep_f32 else t.to(store_dtype)).contiguous().cpu()
     folder = Path(folder)
     folder.mkdir(parents=True, exist_ok=True)
     (folder / "config.json").write_text(json.dumps(config_json, indent=1))

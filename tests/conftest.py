@@ -12,6 +12,17 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X and the built HIP library")
 
 
+def pytest_terminal_summary(terminalreporter):
+    """With -v: how far the bfloat16 comparisons of the run stayed below their bounds."""
+    import traces
+
+    if traces.MEASURED_NOISE and terminalreporter.config.option.verbose > 0:
+        terminalreporter.write_line(f"bfloat16 against plain, {len(traces.MEASURED_NOISE)} comparisons; the largest "
+                                    f"rms and the largest error, in units of the logits' deviation:")
+        for rms, worst, test in sorted(traces.MEASURED_NOISE, reverse=True)[:5]:
+            terminalreporter.write_line(f"  rms {rms:.4f} worst {worst:.4f} {test}")
+
+
 @pytest.fixture(scope="session")
 def tiny_configs():
     """Two tiny configurations that differ in every size and option."""

@@ -24,7 +24,7 @@ def rms_norm(x, weight, eps):
 
 def rope_angles(positions, head_dim, theta):
     """qwen3_runtime/layers/rope.py:18-21: inv = 1/theta^(2j/D); freqs = pos x inv, in float32."""
-    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim)).to(positions.device)
     return positions.to(torch.float32)[:, None] * inv[None, :]  # [T, D/2] float32
 
 
@@ -57,8 +57,8 @@ def causal_attention(q, k, v, scale=None, window=None, q_offset=0):
     k = k.repeat_interleave(g, dim=1)
     v = v.repeat_interleave(g, dim=1)
     scores = torch.einsum("qhd,khd->hqk", q, k) * scale
-    qpos = torch.arange(tq)[:, None] + q_offset
-    kpos = torch.arange(tk)[None, :]
+    qpos = torch.arange(tq, device=q.device)[:, None] + q_offset
+    kpos = torch.arange(tk, device=q.device)[None, :]
     allowed = kpos <= qpos
     if window is not None:
         allowed = allowed & (kpos > qpos - window)
@@ -73,8 +73,10 @@ def swiglu(gate, up):
     return gate * torch.sigmoid(gate) * up
 
 
-def read_model(folder, dtype=torch.float64):
-    """config.json as a dict and every tensor of model.safetensors, upcast to ``dtype``."""
+def read_model(folder, dtype=torch.float64, device="cpu"):
+    """config.json as a dict and every tensor of model.safetensors, upcast to ``dtype``. With a
+    ``device`` the same torch routines run there (the tests of models too large for the host's
+    patience do that); ``forward`` follows the weights' device."""
     from safetensors.torch import load_file
 
     folder = Path(folder)
@@ -82,7 +84,7 @@ def read_model(folder, dtype=torch.float64):
     tensors = {}
     for path in sorted(folder.glob("*.safetensors")):
         tensors.update(load_file(str(path)))
-    return cfg, {k: v.to(dtype) for k, v in tensors.items()}
+    return cfg, {k: v.to(device=device, dtype=dtype) for k, v in tensors.items()}
 
 
 def attention_layer(x, w, prefix, cfg, positions):
@@ -116,8 +118,9 @@ def forward(cfg, w, ids):
     to the embedding or not (tests/cpu/reference_qwen3.py:79-110,
     qwen3_runtime/models/qwen3.py:243-266).
     """
-    ids = torch.as_tensor(ids, dtype=torch.long)
-    positions = torch.arange(ids.numel())
+    dev = w["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(ids, dtype=torch.long, device=dev)
+    positions = torch.arange(ids.numel(), device=dev)
     eps = cfg["rms_norm_eps"]
     h = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):

@@ -52,6 +52,21 @@ def test_cuttings_match_plain(model_folders, tiny_configs, name, cut, dtype):
     check(got, traces.plain_logits(model_folders[name], reqs), dtype)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page", [4, 8, 16])
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_b"])
+def test_page_sizes_under_the_cutting_pattern(model_folders, tiny_configs, name, page, dtype):
+    """Pages of 4, 8 and 16 tokens (the reference's pattern, tests/invariance/test_kv.py:12-69) with
+    requests mixed in a pool at its peak. Pages of 4 are no multiple of 8, so bfloat16 attention
+    then runs in the general kernel instead of the MFMA ones."""
+    cfg, _ = tiny_configs[name]
+    reqs = traces.make_requests(cfg.vocab_size, REUSE_WORKLOADS[name][:6], seed=13)
+    steps = traces.mixed(reqs, seed=page, max_live=3)
+    loaded = load_gpu(model_folders[name], page, traces.peak_tokens(steps, unit=page) // page, dtype)
+    got = traces.replay(loaded, steps)
+    check(got, traces.plain_logits(model_folders[name], reqs), dtype)
+
+
 @pytest.fixture(scope="module")
 def odd_folder(tmp_path_factory):
     """A third tiny model with sizes the kernels' fast paths do not take: head size 80 (a 16-wide

@@ -1,8 +1,13 @@
-"""The engine at the layer sizes of the 4B and 8B models (two layers, a small vocabulary)
-against the plain implementation: the kernels' production paths (few-row products on
-tile-major weights with K cut into planes, the gated epilogue, decode attention at head size
-128 with four query heads per key head, prompt attention through LDS, the vendor products for
-long portions) as parts of a whole model, in float32 and bfloat16."""
+"""The engine at the layer sizes of the 4B, 8B and 32B models (two layers, a small vocabulary; one
+model of the 4B width eight layers deep) against the plain implementation: the kernels'
+production paths (few-row products on tile-major weights with K cut into planes, the gated
+epilogue, decode attention at head size 128 with four and eight query heads per key head, prompt
+attention through LDS, the vendor products for long portions, and at the 32B sizes the same
+without tile-major copies, as that model runs) as parts of a whole model, in float32 and
+bfloat16, under every way of cutting the requests into steps.
+
+Weights of these widths are drawn on the device and the plain implementation's float64 torch
+routines run there too: the host takes minutes for either."""
 
 import dataclasses
 
@@ -13,49 +18,81 @@ import traces
 
 pytestmark = pytest.mark.gpu
 
-# float32: the longest sums have 12,288 terms instead of the tiny models' few hundred.
+# float32: the longest sums have 12,288 (25,600 at the 32B sizes) terms instead of the tiny models' few hundred.
 TOL_F32 = dict(atol=2e-4, rtol=2e-4)
-
+DEVICE = "cuda:0"
+# name -> (preset, layers)
+MODELS = {"qwen3_4b": ("qwen3_4b", 2), "qwen3_8b": ("qwen3_8b", 2), "qwen3_32b": ("qwen3_32b", 2),
+          "deep_4b": ("qwen3_4b", 8)}
+CUTS = ["whole", "tail_one_by_one", "portions", "mixed"]
 
 check_rounding_noise = traces.compare_rounding_noise
 
 
+class _Sized:
+    """Model folders and plain results, made when first asked for and kept for the module."""
+
+    def __init__(self, factory):
+        self.factory = factory
+        self.folders: dict = {}
+        self.plain: dict = {}
+
+    def __getitem__(self, name):
+        if name not in self.folders:
+            from qwen3_runtime_amd.config.presets import preset
+            from qwen3_runtime_amd.weights import write_model_folder
+
+            base, layers = MODELS[name]
+            cfg = dataclasses.replace(preset(base), num_hidden_layers=layers, vocab_size=2048, eos_token_id=None)
+            folder = self.factory.mktemp(name)
+            write_model_folder(folder, cfg.to_dict(), seed=21 + list(MODELS).index(name), device=DEVICE)
+            self.folders[name] = (cfg, folder)
+        return self.folders[name]
+
+    def plain_logits(self, name, lengths, seed, positions=None):
+        key = (name, tuple(lengths), seed, None if positions is None else tuple((r, tuple(p)) for r, p in sorted(positions.items())))
+        if key not in self.plain:
+            cfg, folder = self[name]
+            reqs = traces.make_requests(cfg.vocab_size, lengths, seed=seed)
+            self.plain[key] = (reqs, traces.plain_logits(folder, reqs, device=DEVICE, positions=positions))
+            torch.cuda.empty_cache()
+        return self.plain[key]
+
+
 @pytest.fixture(scope="module")
-def sized_folders(tmp_path_factory):
-    from qwen3_runtime_amd.config.presets import preset
-    from qwen3_runtime_amd.weights import write_model_folder
-
-    out = {}
-    for i, name in enumerate(("qwen3_4b", "qwen3_8b")):
-        cfg = dataclasses.replace(preset(name), num_hidden_layers=2, vocab_size=2048, eos_token_id=None)
-        folder = tmp_path_factory.mktemp(name)
-        write_model_folder(folder, cfg.to_dict(), seed=21 + i)
-        out[name] = (cfg, folder)
-    return out
+def sized(tmp_path_factory):
+    return _Sized(tmp_path_factory)
 
 
-@pytest.fixture(scope="module")
-def plain_results(sized_folders):
-    out = {}
-    for name, (cfg, folder) in sized_folders.items():
-        reqs = traces.make_requests(cfg.vocab_size, [150, 41, 9], seed=6)
-        out[name] = (reqs, traces.plain_logits(folder, reqs))
-    return out
-
-
-@pytest.mark.parametrize("dtype,cut", [("float32", "portions"), ("bfloat16", "mixed"), ("bfloat16", "tail_one_by_one")])
-@pytest.mark.parametrize("name", ["qwen3_4b", "qwen3_8b"])
-def test_model_sized_layers_match_plain(sized_folders, plain_results, name, dtype, cut):
+def load_sized(folder, steps, dtype, *, page=16, copies=True, graph=False, max_seqs=4, pages=None, budget=2048):
     from qwen3_runtime_amd.config.engine import EngineConfig
     from qwen3_runtime_amd.engine.factory import load
 
-    cfg, folder = sized_folders[name]
-    reqs, want = plain_results[name]
+    engine_cfg = EngineConfig(page_size=page, num_pages=pages or -(-traces.peak_tokens(steps) // page),
+                              max_num_seqs=max_seqs, max_num_batched_tokens=budget, dtype=dtype, device=DEVICE,
+                              hip_graph=graph, decode_weight_copy=copies)
+    return load(folder, engine_cfg)
+
+
+def test_the_plain_implementation_is_the_same_on_the_device(model_folders, tiny_configs):
+    """What the comparisons below lean on: the plain implementation run by torch on the device
+    gives the logits it gives on the host (float64 both ways)."""
+    cfg, _ = tiny_configs["tiny_b"]
+    reqs = traces.make_requests(cfg.vocab_size, [70, 9], seed=3)
+    host = traces.plain_logits(model_folders["tiny_b"], reqs)
+    device = traces.plain_logits(model_folders["tiny_b"], reqs, device=DEVICE)
+    traces.compare(device, host, atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", CUTS)
+@pytest.mark.parametrize("name", ["qwen3_4b", "qwen3_8b"])
+def test_model_sized_layers_match_plain(sized, name, cut, dtype):
+    cfg, folder = sized[name]
+    reqs, want = sized.plain_logits(name, [150, 41, 9], seed=6)
     steps = getattr(traces, cut)(reqs)
-    page = 16
-    engine_cfg = EngineConfig(page_size=page, num_pages=traces.peak_tokens(steps) // page, max_num_seqs=4, dtype=dtype,
-                              device="cuda:0", hip_graph=False)
-    loaded = load(folder, engine_cfg)
+    loaded = load_sized(folder, steps, dtype)
+    assert loaded.runner.ops._tiled or dtype == "float32", "the weights have tile-major copies: the own kernels run"
     got = traces.replay(loaded, steps)
     if dtype == "float32":
         traces.compare(got, want, **TOL_F32)
@@ -63,20 +100,41 @@ def test_model_sized_layers_match_plain(sized_folders, plain_results, name, dtyp
         check_rounding_noise(got, want)
 
 
-@pytest.mark.parametrize("live", [20, 40, 64])
-def test_many_requests_decode_together_at_model_sizes(sized_folders, live):
-    """17 to 64 requests decoding in one step at the 4B layer sizes: the products with that many
-    rows (own kernel on tile-major weights: whole result, gated, K cut into planes), decode
-    attention over many sequences. Prompts in three steps, then six steps with a token of every
-    request, against the plain implementation of each request alone."""
-    from qwen3_runtime_amd.config.engine import EngineConfig
-    from qwen3_runtime_amd.engine.factory import load
+@pytest.mark.parametrize("dtype,cut", [("float32", "portions"), ("float32", "tail_one_by_one"), ("bfloat16", "whole"),
+                                       ("bfloat16", "tail_one_by_one"), ("bfloat16", "portions"),
+                                       ("bfloat16", "mixed")])
+def test_32b_layer_sizes_without_decode_copies(sized, dtype, cut):
+    """Width 5,120, 64 query heads on 8 key heads (eight rows of one sequence per decode tile), a
+    feed-forward of 25,600 (the down product's K of 25,600 cut into planes, 1,600 gate/up tiles),
+    and no tile-major copies, as the whole 32B model runs where the copies do not fit: the few-row
+    kernel then reads the weights as stored."""
+    cfg, folder = sized["qwen3_32b"]
+    reqs, want = sized.plain_logits("qwen3_32b", [150, 41, 9], seed=16)
+    steps = getattr(traces, cut)(reqs)
+    loaded = load_sized(folder, steps, dtype, copies=False)
+    assert not loaded.runner.ops._tiled
+    got = traces.replay(loaded, steps)
+    if dtype == "float32":
+        traces.compare(got, want, **TOL_F32)
+    else:
+        check_rounding_noise(got, want)
 
-    cfg, folder = sized_folders["qwen3_4b"]
+
+@pytest.mark.parametrize("name,live,copies", [("qwen3_4b", 20, True), ("qwen3_4b", 40, True), ("qwen3_4b", 64, True),
+                                              ("qwen3_8b", 33, True), ("qwen3_32b", 8, False),
+                                              ("qwen3_32b", 32, False), ("qwen3_32b", 32, True)])
+def test_many_requests_decode_together_at_model_sizes(sized, name, live, copies):
+    """8 to 64 requests decoding in one step at the models' layer sizes: the products with that many
+    rows (own kernel on tile-major weights: whole result, gated, K cut into planes; without the
+    copies the few-row kernel up to 16 rows and the vendor library beyond), decode attention over
+    many sequences. Prompts in three steps, then six steps with a token of every request, against
+    the plain implementation of each request alone."""
+    cfg, folder = sized[name]
     lengths = [9 + (5 * i) % 23 for i in range(live)]
-    reqs = traces.make_requests(cfg.vocab_size, lengths, seed=30 + live)
+    decode = 6
+    reqs, want_all = sized.plain_logits(name, lengths, seed=30 + live)
     rids = list(reqs)
-    steps, decode = [], 6
+    steps = []
     for lo in range(0, live, (live + 2) // 3):
         part = rids[lo: lo + (live + 2) // 3]
         steps.append({"entries": [{"id": r, "tokens": reqs[r][:-decode], "want": [len(reqs[r]) - decode - 1]}
@@ -85,26 +143,21 @@ def test_many_requests_decode_together_at_model_sizes(sized_folders, live):
         steps.append({"entries": [{"id": r, "tokens": reqs[r][len(reqs[r]) - d: len(reqs[r]) - d + 1], "want": [0]}
                                   for r in rids], "end": rids if d == 1 else []})
     steps = traces._number(steps)
-    want_all = traces.plain_logits(folder, reqs)
-    engine_cfg = EngineConfig(page_size=16, num_pages=live * 3, max_num_seqs=live, max_num_batched_tokens=1024,
-                              dtype="bfloat16", device="cuda:0", hip_graph=False)
-    loaded = load(folder, engine_cfg)
-    assert loaded.runner.ops._tiled, "the weights have tile-major copies: the own kernels run"
+    loaded = load_sized(folder, steps, "bfloat16", copies=copies, max_seqs=live, pages=live * 3, budget=1024)
+    assert bool(loaded.runner.ops._tiled) == copies
     got = traces.replay(loaded, steps)
     assert len(got) == live * (decode + 1)
     check_rounding_noise(got, {k: want_all[k] for k in got})
 
 
-def test_long_context_decode_beside_a_prompt_portion(sized_folders, monkeypatch):
+def test_long_context_decode_beside_a_prompt_portion(sized, monkeypatch):
     """Decoded tokens of a request that holds 1,100 keys in the same steps as portions of another
     request's prompt: attention then runs as two launches (the decode kernel with its keys cut
     over blocks, the prompt kernels for the portion). Against the plain implementation."""
-    from qwen3_runtime_amd.config.engine import EngineConfig
-    from qwen3_runtime_amd.engine.factory import load
     from qwen3_runtime_amd.ops.hip import HipOps
 
-    cfg, folder = sized_folders["qwen3_4b"]
-    reqs = traces.make_requests(cfg.vocab_size, [1106, 150], seed=12)
+    cfg, folder = sized["qwen3_4b"]
+    reqs, want = sized.plain_logits("qwen3_4b", [1106, 150], seed=12)
     long_ids, other = reqs["r0"], reqs["r1"]
     steps = [{"entries": [{"id": "r0", "tokens": long_ids[:1100], "want": [1099]}], "end": []}]
     cuts = [0, 40, 70, 100, 120, 137, 150]
@@ -118,15 +171,30 @@ def test_long_context_decode_beside_a_prompt_portion(sized_folders, monkeypatch)
     inner = HipOps._launch_attention
     monkeypatch.setattr(HipOps, "_launch_attention",
                         lambda self, *a: (launches.append(a[-2:]), inner(self, *a))[1])
-    engine_cfg = EngineConfig(page_size=16, num_pages=traces.peak_tokens(steps) // 16, max_num_seqs=4, dtype="bfloat16",
-                              device="cuda:0", hip_graph=False)
-    got = traces.replay(load(folder, engine_cfg), steps)
+    got = traces.replay(load_sized(folder, steps, "bfloat16"), steps)
     assert ([0], True) in launches and ([1], False) in launches, "the mixed steps ran as two launches"
-    want = traces.plain_logits(folder, reqs)
     check_rounding_noise(got, {k: want[k] for k in got})
 
 
-def test_model_sized_decode_graph_equals_eager(sized_folders):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_eight_layers_deep(sized, dtype):
+    """The 4B width eight layers deep, the last 32 tokens of each request decoded one by one from
+    replayed HIP graphs: what the rounding of bfloat16 in every layer adds up to through the
+    float32 residual stays noise of the size the two-layer models show (the bound is the same),
+    and float32 stays at float32's rounding."""
+    cfg, folder = sized["deep_4b"]
+    reqs, want = sized.plain_logits("deep_4b", [150, 41, 36], seed=26)
+    steps = traces.tail_one_by_one(reqs)
+    loaded = load_sized(folder, steps, dtype, graph=True)
+    got = traces.replay(loaded, steps)
+    assert loaded.runner._graphs, "no decode step was replayed from a graph"
+    if dtype == "float32":
+        traces.compare(got, want, **TOL_F32)
+    else:
+        check_rounding_noise(got, want)
+
+
+def test_model_sized_decode_graph_equals_eager(sized):
     """Three requests at the 4B layer sizes, decoded eagerly and then from replayed HIP graphs that
     are fed the eager tokens: at every token the graph's log-probability of it is the eager one up
     to the rounding of bfloat16. (A graph cuts the keys for the length of its bucket, an eager step
@@ -136,7 +204,7 @@ def test_model_sized_decode_graph_equals_eager(sized_folders):
     for the request whose keys are cut differently, 5e-7 for the two that are not.)"""
     from qwen3_runtime_amd.llm import LLM
 
-    cfg, folder = sized_folders["qwen3_4b"]
+    cfg, folder = sized["qwen3_4b"]
     prompts = list(traces.make_requests(cfg.vocab_size, [70, 20, 5], seed=8).values())
 
     def run(graph, forced=None):
@@ -161,24 +229,18 @@ def test_model_sized_decode_graph_equals_eager(sized_folders):
         torch.testing.assert_close(torch.tensor(a), torch.tensor(b), atol=0.03, rtol=0)
 
 
-@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
-def test_the_2048_token_prompt_the_measurement_times(sized_folders, dtype):
-    """One 2,048-token prompt in one step at the 4B layer sizes, the step whose time is reported as
-    prefill throughput: the vendor products at 2,048 rows, the prompt attention through LDS with
-    128 row tiles and their work list, the wide q/k kernel. Logits at every 16th position and at
-    the last ones against the plain implementation."""
-    from qwen3_runtime_amd.config.engine import EngineConfig
-    from qwen3_runtime_amd.engine.factory import load
-
-    cfg, folder = sized_folders["qwen3_4b"]
-    reqs = traces.make_requests(cfg.vocab_size, [2048], seed=44)
-    want_all = traces.plain_logits(folder, reqs)
+@pytest.mark.parametrize("name,dtype,copies", [("qwen3_4b", "bfloat16", True), ("qwen3_4b", "float32", True),
+                                               ("qwen3_32b", "bfloat16", False)])
+def test_the_2048_token_prompt_the_measurement_times(sized, name, dtype, copies):
+    """One 2,048-token prompt in one step, the step whose time is reported as prefill throughput:
+    the vendor products at 2,048 rows, the prompt attention through LDS with 128 (256 at the 32B
+    sizes) row tiles and their work list, the wide q/k kernel. Logits at every 16th position and
+    at the last ones against the plain implementation."""
+    cfg, folder = sized[name]
     wanted = sorted(set(range(0, 2048, 16)) | set(range(2040, 2048)))
+    reqs, want = sized.plain_logits(name, [2048], seed=44, positions={"r0": wanted})
     steps = [{"step": 0, "entries": [{"id": "r0", "tokens": reqs["r0"], "want": wanted}], "end": ["r0"]}]
-    engine_cfg = EngineConfig(page_size=16, num_pages=128, max_num_seqs=1, max_num_batched_tokens=2048, dtype=dtype,
-                              device="cuda:0", hip_graph=False)
-    got = traces.replay(load(folder, engine_cfg), steps)
-    want = {("r0", p): want_all[("r0", p)] for p in wanted}
+    got = traces.replay(load_sized(folder, steps, dtype, copies=copies, max_seqs=1), steps)
     if dtype == "float32":
         traces.compare(got, want, **TOL_F32)
     else:

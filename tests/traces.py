@@ -8,6 +8,7 @@ implementation, whole sequences at once.
 
 from __future__ import annotations
 
+import os
 import random
 
 import torch
@@ -175,21 +176,28 @@ def replay(loaded, steps, check_cache=True, page_users=None):
     return out
 
 
-def plain_logits(folder, requests):
+def plain_logits(folder, requests, device="cpu", positions=None):
+    """The plain implementation's logits by (request, position), float64 arithmetic. ``device``:
+    where torch runs it (models of a real width take minutes on the host); ``positions``: keep
+    these only, per request."""
     from plain import qwen3_plain as P
 
-    cfg, w = P.read_model(folder)
+    cfg, w = P.read_model(folder, device=device)
     out = {}
     for rid, toks in requests.items():
-        logits = P.forward(cfg, w, toks)
-        for p in range(len(toks)):
-            out[(rid, p)] = logits[p].float()
+        logits = P.forward(cfg, w, toks).float().cpu()
+        for p in (range(len(toks)) if positions is None else positions[rid]):
+            out[(rid, p)] = logits[p]
     return out
 
 
 def make_requests(vocab, lengths, seed=0):
     g = torch.Generator().manual_seed(seed)
     return {f"r{i}": torch.randint(0, vocab, (n,), generator=g).tolist() for i, n in enumerate(lengths)}
+
+
+# (rms, worst) of every bfloat16 comparison of the run, in units of the logits' deviation
+MEASURED_NOISE: list = []
 
 
 def compare_rounding_noise(got, want, rms_bound=0.015, worst_bound=0.08):
@@ -213,6 +221,7 @@ def compare_rounding_noise(got, want, rms_bound=0.015, worst_bound=0.08):
         f"largest error {worst:.4f} at (request, position) {where}; logit deviation {std:.3f}; "
         f"first position over the bound: {over[0]}")
     assert rms < rms_bound * std, f"rms error {rms:.4f} against a logit deviation of {std:.3f}"
+    MEASURED_NOISE.append((rms / std, worst / std, os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0]))
     return rms / std, worst / std
 
 
