@@ -98,12 +98,17 @@ constexpr int DB = D / 16;           // 16-wide blocks of the head dimension
 template <bool P2> __device__ __forceinline__ int page_div(int x, int ps, int shift) { return P2 ? x >> shift : x / ps; }
 template <bool P2> __device__ __forceinline__ int page_mod(int x, int ps) { return P2 ? x & (ps - 1) : x % ps; }
 
-// ``v`` if ``keep``, else zeros: four 32-bit selects (element by element it was sixteen
-// instructions with the shifts and packs around them)
-__device__ __forceinline__ bf16x8_t keep_or_zero(bf16x8_t v, bool keep) {
+// The first ``n`` of the 8 values of ``v`` (n <= 0: none, n >= 8: all), zeros for the others:
+// four masks made once per group of keys and four ANDs per operand. A group of 8 keys that
+// straddles the last key any row of the block of waves sees holds, after it, places nobody has
+// written since the page's last holder: their probabilities are zero, but 0 x NaN is NaN, so
+// the values themselves become zeros, key by key.
+__device__ __forceinline__ bf16x8_t keep_first(bf16x8_t v, int n) {
   typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-  const u32x4_t bits = __builtin_bit_cast(u32x4_t, v);
-  return __builtin_bit_cast(bf16x8_t, keep ? bits : (u32x4_t){0u, 0u, 0u, 0u});
+  u32x4_t bits = __builtin_bit_cast(u32x4_t, v);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) bits[j] &= n >= 2 * j + 2 ? 0xffffffffu : (n == 2 * j + 1 ? 0x0000ffffu : 0u);
+  return __builtin_bit_cast(bf16x8_t, bits);
 }
 
 // The larger of two, a NaN if either is one (IEEE 754-2019 maximum): one instruction, where
@@ -353,12 +358,13 @@ __global__ __launch_bounds__(256, RT <= 2 ? 2 : 1) void attention_bf16_kernel(At
       KvBlock blk;
       block_load<P2>(a, kvh, base, lo, pos_max, r16, quad, pg, blk);
       block_pages<P2>(table, min(b + 1, b1 - 1) << 5, lo, pos_max, ps, r16, quad, pg_next);
-      // values of keys outside [lo, pos_max] came from a clamped place and may be anything
+      // values of keys outside [lo, pos_max] came from a clamped place, or from places after the
+      // sequence's last key in its last page, and may be anything
       const int kv0 = base + 8 * quad;
       if (base < lo || base + 31 > pos_max) {  // the same for the whole wave
-        const bool seen = kv0 <= pos_max && kv0 + 7 >= lo;
+        const int keep = kv0 + 7 >= lo ? pos_max - kv0 + 1 : 0;
 #pragma unroll
-        for (int i = 0; i < DB; ++i) blk.v[i] = keep_or_zero(blk.v[i], seen);
+        for (int i = 0; i < DB; ++i) blk.v[i] = keep_first(blk.v[i], keep);
       }
 #pragma unroll
       for (int t = 0; t < RT; ++t) {
@@ -581,10 +587,11 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   auto stash = [&](int b, int stage, const Pieces& in) {  // registers -> LDS: block b into its stage
     bf16_t* kb = lds_kv + stage * STAGE_ELEMS;
     bf16_t* vb = kb + 32 * KROW;
-    // values of keys no row of the block sees were read from a clamped place: they may be
-    // anything, and 0 * NaN is NaN, so they become zeros
+    // values of keys no row of the block sees were read from a clamped place, or lie after the
+    // sequence's last key in its last page: they may be anything, and 0 * NaN is NaN, so they
+    // become zeros
     const int g0 = (b << 5) + w8;
-    const bool seen = g0 <= blk_pos_max && g0 + 7 >= lo;
+    const int keep = g0 + 7 >= lo ? blk_pos_max - g0 + 1 : 0;
 #pragma unroll
     for (int i = 0; i < LANE_PIECES; ++i) {
       const int c = lane + 64 * i;
@@ -596,7 +603,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
         const int kl = c / (D / 8), part = c - kl * (D / 8);
         const int row = 16 * (kl >> 2) + (w8 >> 1) + (kl & 3);
         *(bf16x8_t*)(kb + row * KROW + 8 * part) = in.k[i];
-        *(bf16x8_t*)(vb + c * VROW + w8) = keep_or_zero(in.v[i], seen);
+        *(bf16x8_t*)(vb + c * VROW + w8) = keep_first(in.v[i], keep);
       }
     }
   };
@@ -833,11 +840,12 @@ __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg
   // the same for the whole wave: does every row see all 32 keys?
   const bool whole = base + 31 <= pos_min && (window == 0 || base > pos_max - window);
   if (!whole) {
-    // values of keys outside [lo, pos_max] came from a clamped place and may be anything
+    // values of keys outside [lo, pos_max] came from a clamped place, or from places after the
+    // sequence's last key in its last page, and may be anything
     const int kv0 = base + 8 * quad;
-    const bool seen = kv0 <= pos_max && kv0 + 7 >= lo;
+    const int keep = kv0 + 7 >= lo ? pos_max - kv0 + 1 : 0;
 #pragma unroll
-    for (int i = 0; i < DB; ++i) blk.v[i] = keep_or_zero(blk.v[i], seen);
+    for (int i = 0; i < DB; ++i) blk.v[i] = keep_first(blk.v[i], keep);
   }
   tile_update(s, blk.v, !whole, base, quad, row_valid, qpos, window, scale_log2, m, l, o);
 }

@@ -118,6 +118,21 @@ def test_mixed_with_page_reuse(model_folders, tiny_configs, name, dtype):
     check(got, traces.plain_logits(model_folders[name], reqs), dtype)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_b"])
+def test_pages_that_come_back_full_of_nan(model_folders, tiny_configs, name, dtype):
+    """The same with every page filled with NaN and infinities at the start and again whenever its
+    request ends: a later holder writes its own keys and values into part of such a page, and the
+    places it has not written yet (the rest of the page, within the last group of 8 keys too)
+    must not be multiplied, not even by a probability of zero."""
+    cfg, page = tiny_configs[name]
+    reqs = traces.make_requests(cfg.vocab_size, REUSE_WORKLOADS[name], seed=19)
+    steps = traces.mixed(reqs, seed=4, max_live=3 if name == "tiny_a" else 4)
+    loaded = load_gpu(model_folders[name], page, traces.peak_tokens(steps, unit=page) // page, dtype)
+    got = traces.replay(loaded, steps, poison_freed=True)
+    check(got, traces.plain_logits(model_folders[name], reqs), dtype)
+
+
 @pytest.mark.parametrize("seed", [3, 5, 6, 17, 26, 45])
 def test_random_models_and_random_traces(tmp_path, seed):
     """A model and a trace drawn from the seed: head sizes 16 to 256 (64 and up also take the decode

@@ -381,8 +381,11 @@ def test_qk_norm_rope_store_neighbouring_slots(ops, dtype, t, nq, nkv, d, ps, st
     close(cache.v, want_cache.v, 0, 0)
 
 
-def build_attention_case(seqs, nq, nkv, d, ps, dtype, seed=0, window=None, shuffle=True, spare_pages=3):
-    """seqs: list of (q_len, kv_len). Returns q, cache view with filled pages, ctx."""
+def build_attention_case(seqs, nq, nkv, d, ps, dtype, seed=0, window=None, shuffle=True, spare_pages=3,
+                         poison=False):
+    """seqs: list of (q_len, kv_len). Returns q, cache view with filled pages, ctx. ``poison``:
+    every place no sequence has written (the rest of each sequence's last page, pages in no
+    table) holds NaN or an infinity instead of noise, as a page's last holder may have left."""
     from qwen3_runtime_amd.parts.base import StepContext
 
     g = torch.Generator().manual_seed(seed)
@@ -399,6 +402,16 @@ def build_attention_case(seqs, nq, nkv, d, ps, dtype, seed=0, window=None, shuff
         n = (kv + ps - 1) // ps
         table[s, :n] = order[nxt: nxt + n].to(torch.int32)
         nxt += n
+    if poison:
+        written = torch.zeros(total_pages, ps, dtype=torch.bool)
+        for s, (_, kv) in enumerate(seqs):
+            pos = torch.arange(kv)
+            written[table[s, pos // ps].long(), pos % ps] = True
+        bad = torch.tensor([float("nan"), float("inf"), float("-inf")])[torch.arange(total_pages * ps) % 3]
+        bad = bad.view(total_pages, ps).to(dtype).to(DEV)
+        unwritten = (~written).to(DEV)
+        cache.k.copy_(torch.where(unwritten[:, None, :, None], bad[:, None, :, None], cache.k))
+        cache.v.copy_(torch.where(unwritten[:, None, None, :], bad[:, None, None, :], cache.v))
     t = sum(q for q, _ in seqs)
     q = (torch.randn(t, nq * d, generator=g)).to(dtype).to(DEV)
     cu = [0]
@@ -449,6 +462,32 @@ def test_paged_attention(ops, dtype, seqs, nq, nkv, d, ps):
     got = ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, None)
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     close(got, want, tol, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("seqs,nq,nkv,d,ps", [
+    ([(7, 7), (1, 41), (33, 35), (1, 1)], 4, 2, 16, 16),     # general kernel; decode kernel for the single tokens alone
+    ([(1, 300), (1, 17), (1, 61), (1, 67)], 8, 2, 64, 8),    # decode kernel, several key splits
+    ([(150, 213), (70, 70)], 4, 1, 128, 16),                 # long portions through LDS
+    ([(100, 1501)], 8, 2, 64, 32),                           # ... with the keys cut over blocks
+    ([(1, 1203), (90, 91)], 32, 8, 128, 16),                 # two launches
+    ([(150, 211)], 2, 1, 256, 16),                           # general kernel with two row tiles
+])
+def test_paged_attention_ignores_what_a_page_held_before(ops, dtype, seqs, nq, nkv, d, ps):
+    """Every place of the cache that the sequences have not written holds NaN or an infinity: the
+    rest of each last page (within the last group of 8 keys and after it) and every page in no
+    table. A kernel that multiplies such a value, by a probability of zero too, shows it."""
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, dtype, poison=True)
+    scale = 1.0 / math.sqrt(d)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, scale)
+    assert torch.isfinite(want.float()).all()
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    close(ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, None), want, tol, tol)
+    if dtype == torch.bfloat16:
+        for splits in (2, 5):
+            ctx.scratch["attn_splits"] = splits
+            close(ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, None), want, tol, tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -521,6 +560,40 @@ def test_decode_attention_with_the_tokens_own_key_from_the_product(ops, nq, nkv,
         cache.k.copy_(before_k)
         cache.v.copy_(before_v)
         ctx.scratch["attn_splits"] = splits
+        close(ops.decode_attention(qkv, cache, ctx, nq, nkv, d, scale, window, qw, kw, 1e-6, inv), want, 2e-2, 2e-2)
+
+
+@pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, None), (8, 2, 64, 8, None), (8, 2, 64, 16, 40)])
+def test_decode_attention_ignores_what_a_page_held_before(ops, nq, nkv, d, ps, window):
+    """The one-kernel decode step with NaN and infinities in every place of the cache no sequence
+    has written, the tokens' own places included (the kernel fills them; it must not read them)."""
+    kvs = [1, 2, 9, 32, 33, 41, 64, 65, 300, 2100, ps, ps + 1]
+    seqs = [(1, kv) for kv in kvs]
+    _, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, window=window, seed=4, poison=True)
+    t = len(seqs)
+    qkv = rnd(t, (nq + 2 * nkv) * d, dtype=torch.bfloat16, seed=12)
+    qw, kw = 1 + 0.1 * rnd(d, seed=5), 1 + 0.1 * rnd(d, seed=6)
+    inv = (1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    table = cache.group.block_table.cpu()
+    slots = torch.tensor([int(table[i, (kv - 1) // ps]) * ps + (kv - 1) % ps for i, kv in enumerate(kvs)],
+                         dtype=torch.int32, device=DEV)
+    cache.group.slots = slots
+    pages, offs = (slots // ps).long(), (slots % ps).long()
+    cache.k[pages, :, offs, :] = float("nan")
+    cache.v[pages, :, :, offs] = float("inf")
+    before_k, before_v = cache.k.clone(), cache.v.clone()
+    scale = 1.0 / math.sqrt(d)
+    want_k, want_v = cache.k.clone(), cache.v.clone()
+    q = R.qk_norm_rope_store(qkv, nq, nkv, d, qw, kw, 1e-6, inv, ctx.positions, want_k, want_v, slots, ps)
+    want = R.paged_attention(q.to(torch.bfloat16), want_k, want_v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(),
+                             cache.group.block_table, ps, nq, nkv, d, scale, window)
+    assert torch.isfinite(want.float()).all()
+    for splits in (None, 1, 3):
+        cache.k.copy_(before_k)
+        cache.v.copy_(before_v)
+        ctx.scratch.pop("attn_splits", None)
+        if splits:
+            ctx.scratch["attn_splits"] = splits
         close(ops.decode_attention(qkv, cache, ctx, nq, nkv, d, scale, window, qw, kw, 1e-6, inv), want, 2e-2, 2e-2)
 
 

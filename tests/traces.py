@@ -138,14 +138,24 @@ def peak_tokens(steps, unit=64):
     return peak
 
 
-def replay(loaded, steps, check_cache=True, page_users=None):
+def replay(loaded, steps, check_cache=True, page_users=None, poison_freed=False):
     """Run the steps through ``loaded.runner``; returns {(request, position): logits row}.
-    ``page_users`` (a dict) receives, per page of the first cache group, the requests that held it."""
+    ``page_users`` (a dict) receives, per page of the first cache group, the requests that held it.
+    ``poison_freed``: the pages a request gives back are filled with NaN (keys) and infinities
+    (values) before anyone takes them again, and so are all pages before the first step."""
     from qwen3_runtime_amd.engine.batch import StepEntry
 
     runner, cache = loaded.runner, loaded.cache
     pos: dict[str, int] = {}
     out = {}
+
+    def poison(group, pages):
+        group.storage[:, 0, pages] = float("nan")
+        group.storage[:, 1, pages] = float("inf")
+
+    if poison_freed:
+        for g in cache.groups:
+            poison(g, slice(None))
     for s in steps:
         entries = []
         for e in s["entries"]:
@@ -169,7 +179,11 @@ def replay(loaded, steps, check_cache=True, page_users=None):
                     if page >= 0:
                         page_users.setdefault(page, set()).add(e["id"])
         for rid in s["end"]:
+            held = [[p for p in g.tables[rid] if p >= 0] for g in cache.groups]
             cache.release(rid)
+            if poison_freed:
+                for g, pages in zip(cache.groups, held):
+                    poison(g, torch.tensor(pages, dtype=torch.long, device=g.storage.device))
         if check_cache:
             cache.check()
     assert not cache.live_requests()
