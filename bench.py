@@ -92,6 +92,15 @@ def measure_device_peaks(device) -> dict:
             "mfma_bf16_tflops": round(blocks * 4 * iters * 4 * 32768 / t_mfma / 1e12, 1)}
 
 
+def sizes_of(raw: dict, limit: int = 12) -> dict:
+    """The sizes and switches of a config.json: its integer and boolean entries, without the
+    ids of special tokens and the position limit (no sizes of the computation)."""
+    skip = ("token_id", "max_position", "max_window", "seed")
+    out = {k: v for k, v in raw.items()
+           if isinstance(v, (bool, int)) and not any(s in k for s in skip) and (v is not False or k.startswith("tie"))}
+    return dict(list(out.items())[:limit])
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -118,17 +127,19 @@ def main() -> int:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine is single-GPU)")
         return 2
 
-    import dataclasses
-
     import torch
 
-    from qwen3_runtime_amd.config.presets import preset
     from qwen3_runtime_amd.engine.batch import StepEntry
     from qwen3_runtime_amd.llm import build_engine
+    from qwen3_runtime_amd.registry import preset_config
     from qwen3_runtime_amd.sampling.params import SamplingParams
 
-    cfg_full = preset(args.preset)
-    cfg = cfg_full if args.layers is None else dataclasses.replace(cfg_full, num_hidden_layers=args.layers)
+    # the configuration is a config.json as a dict; nothing below knows which architecture it names:
+    # bytes and operations of a step come from the model's parts and the cache manager
+    raw_full = preset_config(args.preset)
+    raw = dict(raw_full)
+    if args.layers is not None:
+        raw["num_hidden_layers"] = args.layers
     steps, warmup, trials = args.steps, args.warmup, max(1, args.trials)
     page = 16
     max_batch = args.batch if (args.no_points or args.prefill_only) else max(args.batch, 64)
@@ -153,7 +164,7 @@ def main() -> int:
         pages = max_batch * (-(-(4096 + 256) // page) + 1)
     t0 = time.time()
     engine = build_engine(
-        None, config=cfg, seed=20260825, dtype=args.dtype, block_size=page, num_kv_blocks=pages,
+        None, config=raw, seed=20260825, dtype=args.dtype, block_size=page, num_kv_blocks=pages,
         max_num_seqs=max_batch, max_num_batched_tokens=budget, max_model_len=args.context,
         cuda_graph=not args.no_graph,
     )
@@ -162,17 +173,18 @@ def main() -> int:
     dev = engine.runner.device
     gen = torch.Generator().manual_seed(20260825)
     bytes_el = 2 if args.dtype == "bfloat16" else 4
-    kv_bytes_per_token = 2 * cfg.num_hidden_layers * cfg.kv_width * bytes_el
-    # every weight a step uses, once: a tied table is read once, as the head; an untied
-    # embedding table is only looked up
-    head_bytes = cfg.vocab_size * cfg.hidden_size * bytes_el
-    step_weight_bytes = engine.loaded.weight_bytes - (0 if cfg.tie_word_embeddings else head_bytes)
-    linear_flop_per_token = 2 * cfg.num_hidden_layers * (
-        cfg.hidden_size * (cfg.q_width + 2 * cfg.kv_width) + cfg.q_width * cfg.hidden_size
-        + 3 * cfg.hidden_size * cfg.intermediate_size)
+    model, vocab = engine.loaded.model, engine.loaded.model.plan.vocab_size
 
-    def roofline(step_seconds: float, kv_tokens: float) -> dict:
-        achieved = (step_weight_bytes + kv_tokens * kv_bytes_per_token) / step_seconds / 1e9
+    def step_bytes_and_flop(spans, rows):
+        """What a step over ``spans`` = (tokens of the step, tokens in the cache after it) has to
+        read (every weight it uses once: a table that is only looked up counts its rows; and the
+        cache of its requests) and to compute, as the model's parts and the cache manager say."""
+        cost = model.step_cost(spans, rows, bytes_el)
+        return cost.total_weight_bytes + engine.cache.bytes_read([kv for _, kv in spans], bytes_el), cost.flop
+
+    def roofline(step_seconds: float, kv_lens) -> dict:
+        nbytes, _ = step_bytes_and_flop([(1, round(kv)) for kv in kv_lens], len(kv_lens))
+        achieved = nbytes / step_seconds / 1e9
         out = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                "frac": round(achieved / HBM_PEAK_GBS, 4)}
         if peaks:
@@ -182,9 +194,9 @@ def main() -> int:
 
     def decode_run(batch: int, k: int, w: int, n_trials: int):
         """Read ``batch`` prompts in, then ``n_trials`` windows of ``k`` timed decode steps after ``w``
-        warm-up steps. Returns the windows as (seconds, mean tokens in the cache), and the time the
-        prompts took."""
-        prompts = torch.randint(0, cfg.vocab_size, (batch, args.prompt_len), generator=gen).tolist()
+        warm-up steps. Returns the windows as (seconds, tokens each request holds at the window's
+        middle), and the time the prompts took."""
+        prompts = torch.randint(0, vocab, (batch, args.prompt_len), generator=gen).tolist()
         reqs = [engine.request(engine.add_request(p, max_tokens=n_trials * k + w + lead(batch) + 8,
                                                   sampling=SamplingParams())) for p in prompts]
         torch.cuda.synchronize(dev)
@@ -198,15 +210,15 @@ def main() -> int:
         windows = []
         for _ in range(n_trials):
             torch.cuda.synchronize(dev)
-            kv_before = sum(engine.cache.length(r.request_id) for r in reqs)
+            kv_before = [engine.cache.length(r.request_id) for r in reqs]
             t = time.perf_counter()
             for _ in range(k):
                 out = engine.step()
                 assert len(out) == batch and all(tok is not None for _, tok, _ in out)
             torch.cuda.synchronize(dev)
             dt = time.perf_counter() - t
-            kv_after = sum(engine.cache.length(r.request_id) for r in reqs)
-            windows.append((dt, (kv_before + kv_after) / 2))
+            kv_after = [engine.cache.length(r.request_id) for r in reqs]
+            windows.append((dt, [(a + b) / 2 for a, b in zip(kv_before, kv_after)]))
         for r in reqs:
             engine.finish_request(r.request_id)
         return windows, fill
@@ -217,7 +229,7 @@ def main() -> int:
     def prefill_run():
         """One 2,048-token prompt through the step function, logits at its last token."""
         tokens = 2048
-        ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=gen).tolist()
+        ids = torch.randint(0, vocab, (tokens,), generator=gen).tolist()
         times = []
         for i in range(1 + trials):
             rid = f"prefill{i}"
@@ -230,9 +242,7 @@ def main() -> int:
             engine.cache.release(rid)
         timed = times[1:]  # the first is the warm-up
         pt = statistics.median(timed)
-        attn = 2 * cfg.q_width * tokens * tokens * cfg.num_hidden_layers
-        head = 2 * cfg.vocab_size * cfg.hidden_size
-        flop = linear_flop_per_token * tokens + attn + head
+        _, flop = step_bytes_and_flop([(tokens, tokens)], 1)
         peak = MFMA_PEAK[dtype_key]
         out = {"value": round(tokens / pt, 1), "tokens": tokens, "ms": round(pt * 1e3, 3),
                "frac": round(flop / pt / peak, 4), "trials": len(timed), "spread": spread(timed)}
@@ -249,7 +259,7 @@ def main() -> int:
         # continuous batching: every request queued at once, prompts read in portions beside the
         # decoding of those already in
         lengths = torch.randint(128, 4097, (args.requests,), generator=gen).tolist()
-        prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for n in lengths]
+        prompts = [torch.randint(0, vocab, (n,), generator=gen).tolist() for n in lengths]
         engine.generate_batch(prompts[:2], max_tokens=8)  # warm-up: libraries, allocator
         torch.cuda.synchronize(dev)
         t = time.perf_counter()
@@ -261,10 +271,8 @@ def main() -> int:
             out = engine.step()
             now = time.perf_counter() - t
             stats = engine.last_step_stats
-            step_tokens = stats["prefill_tokens"] + stats["decode_tokens"]
-            kv_read = sum(engine.cache.length(rid) for rid in stats["req_ids"] if engine.cache.has(rid))
-            floor_s += max((step_weight_bytes + kv_read * kv_bytes_per_token) / (HBM_PEAK_GBS * 1e9),
-                           linear_flop_per_token * step_tokens / MFMA_PEAK[dtype_key])
+            nbytes, flop = step_bytes_and_flop(stats["spans"], sum(tok is not None for _, tok, _ in out))
+            floor_s += max(nbytes / (HBM_PEAK_GBS * 1e9), flop / MFMA_PEAK[dtype_key])
             for rid, tok, _done in out:
                 if tok is not None:
                     stamps[rid].append(now)
@@ -292,7 +300,7 @@ def main() -> int:
             "measured_peak": peaks,
             "preemptions": engine.scheduler.num_preemptions, "dtype": dtype_key,
             "data": "synthetic: uniform-random token ids and lengths, seeded random weights",
-            "config": {"model": f"{args.preset} shape", "layers": cfg.num_hidden_layers, "max_num_seqs": max_batch,
+            "config": {"model": f"{args.preset} shape", "layers": len(model.plan.order), "max_num_seqs": max_batch,
                        "max_num_batched_tokens": budget, "page_size": page, "hip_graph": not args.no_graph},
         }), flush=True)
         return 0
@@ -331,15 +339,9 @@ def main() -> int:
         "data": "synthetic: uniform-random token ids, seeded random weights N(0, 0.02), norms 1.0",
         "config": {
             "model": f"{args.preset} shape",
-            "layers": cfg.num_hidden_layers,
-            "layers_of_full_model": cfg_full.num_hidden_layers,
-            "hidden": cfg.hidden_size,
-            "heads": cfg.num_attention_heads,
-            "kv_heads": cfg.num_key_value_heads,
-            "head_dim": cfg.head_dim,
-            "intermediate": cfg.intermediate_size,
-            "vocab": cfg.vocab_size,
-            "tied_head": cfg.tie_word_embeddings,
+            # every size of the configuration, under config.json's own names
+            **sizes_of(raw),
+            "layers_of_full_model": raw_full.get("num_hidden_layers", len(model.plan.order)),
             "global_batch": args.batch,
             "seq_len": args.prompt_len,
             "context_limit": args.context,

@@ -14,9 +14,12 @@ the step's tokens; reference: qwen3_runtime/engine/block_manager.py:85-95) and
 later query can see), finally ``release``. ``restart`` drops the pages but
 keeps the slot, for a request that is preempted and recomputed.
 
-Device layout of a paged cache: keys ``[page, head, offset, D]``, values
-``[page, head, D, offset]`` (values transposed inside a page, so that the
-attention kernels read keys-contiguous operands for both products).
+Device layout of a paged cache: one tensor per ``PagedStream`` of its spec,
+``[page, head, offset, width]`` or, transposed, ``[page, head, width, offset]``.
+Keys and values (``"paged_kv"``) are the streams ``k`` and ``v``, the values
+transposed inside a page, so that the attention kernels read keys-contiguous
+operands for both products; a mixer that keeps something else per token (values of
+another width than its keys, one latent vector) names its own streams.
 """
 
 from __future__ import annotations
@@ -44,7 +47,8 @@ class _Group:
     tables: dict[Hashable, list[int]] = field(default_factory=dict)
     # index of the first table entry that still holds a page
     first_live: dict[Hashable, int] = field(default_factory=dict)
-    storage: torch.Tensor | None = None
+    # per stream of the spec: [caches of the group, pages, elements of the stream per page]
+    storage: list[torch.Tensor] | None = None
 
     def pages_for(self, length: int) -> int:
         return (length + self.page_size - 1) // self.page_size if length > 0 else 0
@@ -78,7 +82,7 @@ class CacheManager:
         self.epoch = 0
         by_key: dict[tuple, _Group] = {}
         for cid, spec in enumerate(self.specs):
-            if spec.kind == "paged_kv":
+            if spec.paged:
                 key = spec.group_key()
                 if key not in by_key:
                     by_key[key] = _Group(key, spec, [], PagePool(num_pages), self.page_size, spec.window)
@@ -92,10 +96,11 @@ class CacheManager:
                 raise ValueError(f"unknown cache kind {spec.kind!r}")
         if allocate:
             for g in self.groups:
-                per_page = g.spec.heads * self.page_size * g.spec.head_dim
-                g.storage = torch.zeros(
-                    (len(g.cache_ids), 2, g.pool.num_pages, per_page), dtype=dtype, device=self.device
-                )
+                g.storage = [
+                    torch.zeros((len(g.cache_ids), g.pool.num_pages, stream.elements_per_token() * self.page_size),
+                                dtype=dtype, device=self.device)
+                    for stream in g.spec.page_streams()
+                ]
 
     # ---- sizes -------------------------------------------------------------
     @staticmethod
@@ -105,9 +110,21 @@ class CacheManager:
         4B shape, bfloat16, 16 tokens: 2*36*8*128*2*16 = 2,359,296
         (reference: qwen3_runtime/engine/memory.py:8-14).
         """
-        return sum(
-            2 * s.heads * s.head_dim * page_size * dtype_bytes for s in specs if s.kind == "paged_kv"
-        )
+        return sum(s.elements_per_token() * page_size * dtype_bytes for s in specs if s.paged)
+
+    def bytes_read(self, kv_lens: Sequence[int], dtype_bytes: int | None = None) -> int:
+        """Bytes of cache a step has to read for requests that hold ``kv_lens`` tokens: every
+        stream of every paged cache for the tokens a query still sees (all of them, or the
+        last ``window``), and every fixed-size state once per request."""
+        width = dtype_bytes or torch.finfo(self.dtype).bits // 8
+        total = 0
+        for spec in self.specs:
+            if spec.paged:
+                seen = sum(n if spec.window is None else min(n, spec.window) for n in kv_lens)
+                total += seen * spec.elements_per_token() * width
+        for state in self._state_of_cache.values():
+            total += len(kv_lens) * state[0].numel() * state.element_size()
+        return total
 
     @property
     def num_pages(self) -> int:
@@ -119,6 +136,22 @@ class CacheManager:
 
     def pages_needed_for(self, length: int) -> int:
         return (length + self.page_size - 1) // self.page_size if length > 0 else 0
+
+    def can_ever_hold(self, length: int) -> tuple[bool, str]:
+        """Whether a request that grows to ``length`` tokens fits the pools when it runs alone,
+        one token a step if need be: a group that keeps all keys needs the pages of ``length``
+        tokens, a window group only the pages its window can touch (it gives the others back as
+        it goes). Returns (fits, why not)."""
+        for i, g in enumerate(self.groups):
+            need = g.pages_for(length)
+            if g.window is not None:
+                # `window` consecutive positions touch at most this many pages
+                need = min(need, (g.window - 1 + g.page_size - 1) // g.page_size + 1)
+            if need > g.pool.num_pages:
+                what = "" if g.window is None else f" (window {g.window})"
+                return False, (f"request length {length} needs {need} cache pages in group {i}{what}; "
+                               f"the pool has {g.pool.num_pages}")
+        return True, ""
 
     # ---- request lifetime --------------------------------------------------
     def has(self, rid: Hashable) -> bool:
@@ -291,6 +324,6 @@ class CacheManager:
         g = self.groups[gi]
         i = g.cache_ids.index(cache_id)
         n = g.pool.num_pages
-        k = g.storage[i, 0].view(n, spec.heads, g.page_size, spec.head_dim)
-        v = g.storage[i, 1].view(n, spec.heads, spec.head_dim, g.page_size)
-        return CacheView(spec, writes=writes, group=group_views[gi], k=k, v=v)
+        pages = {stream.name: store[i].view(n, *stream.page_shape(g.page_size))
+                 for stream, store in zip(spec.page_streams(), g.storage)}
+        return CacheView(spec, writes=writes, group=group_views[gi], k=pages.get("k"), v=pages.get("v"), pages=pages)

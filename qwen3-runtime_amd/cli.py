@@ -41,7 +41,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
     args = ap.parse_args(argv)
 
-    from .config.presets import preset
+    from .registry import preset_config
     from .sampling.params import SamplingParams
 
     if args.write_model:
@@ -49,7 +49,7 @@ def main(argv=None) -> int:
             ap.error("--write-model needs --preset")
         from .weights import write_model_folder
 
-        print("wrote", write_model_folder(args.write_model, preset(args.preset).to_dict(), args.seed))
+        print("wrote", write_model_folder(args.write_model, preset_config(args.preset), args.seed))
         return 0
     if not args.model and not args.preset:
         raise SystemExit("set --model or QWEN3_RUNTIME_MODEL (or --preset for random weights)")
@@ -59,7 +59,7 @@ def main(argv=None) -> int:
 
     engine = build_engine(
         args.model if not args.preset else None,
-        config=preset(args.preset) if args.preset else None, seed=args.seed,
+        config=preset_config(args.preset) if args.preset else None, seed=args.seed,
         max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
         block_size=args.block_size, num_kv_blocks=args.num_kv_blocks, dtype=args.dtype,
         cuda_graph=args.cuda_graph,

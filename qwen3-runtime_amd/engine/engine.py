@@ -107,7 +107,7 @@ class Engine:
                    for r in batch)
 
     def _run_step(self, batch: list[Request], evictions_before: int):
-        entries, to_sample = [], []
+        entries, to_sample, spans = [], [], []
         n_prompt = n_decode = 0
         for req in batch:
             at = self.cache.length(req.request_id)
@@ -116,6 +116,7 @@ class Engine:
                                    req.token_ids[: req.prompt_len])
             upto = at + req.grant
             caught_up = upto >= len(req.token_ids)
+            spans.append((req.grant, upto))
             entries.append(StepEntry(req.request_id, req.token_ids[at:upto], [req.grant - 1] if caught_up else []))
             if caught_up:
                 to_sample.append(req)
@@ -144,6 +145,7 @@ class Engine:
             self._live.pop(rid, None)
         self.last_step_stats = {
             "req_ids": [req.request_id for req in batch],
+            "spans": spans,  # per request: (tokens of the step, tokens in the cache after it)
             "prefill_tokens": n_prompt,
             "decode_tokens": n_decode,
             "preempts": self.scheduler.num_preemptions - evictions_before,

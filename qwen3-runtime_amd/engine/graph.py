@@ -240,5 +240,5 @@ class DecodeGraph:
         return self.logits
 
     def _min_kv_heads(self) -> int:
-        heads = [s.heads for s in self.runner.model.plan.caches if s.kind == "paged_kv"]
+        heads = [stream.heads for s in self.runner.model.plan.caches for stream in s.page_streams()]
         return min(heads) if heads else 1

@@ -50,7 +50,7 @@ class ModelRunner:
         # A step may be launched before it is asked for, and then not be asked for after all, only
         # if running it has no effect that a later step could see: keys and values written beyond
         # a request's counted length are such; a per-request state that the step replaces is not.
-        self.repeatable = all(s.kind == "paged_kv" for s in model.plan.caches)
+        self.repeatable = all(s.paged for s in model.plan.caches)
         self.steps_ahead = [0, 0]  # launched before they were asked for; of these, asked for
 
     # ---- public ------------------------------------------------------------

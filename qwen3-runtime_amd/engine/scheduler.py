@@ -52,10 +52,10 @@ class Scheduler:
         if longest - 1 > self.max_model_len:
             raise RuntimeError(
                 f"request length {longest} exceeds the model's limit of {self.max_model_len} positions")
-        pages = self.cache.pages_needed_for(longest)
-        if self.cache.groups and pages > self.cache.num_pages:
-            raise RuntimeError(
-                f"request length {longest} needs {pages} cache pages; the pool has {self.cache.num_pages}")
+        # per group of caches: one that keeps a window of keys needs the window's pages only
+        fits, why_not = self.cache.can_ever_hold(longest)
+        if not fits:
+            raise RuntimeError(why_not)
         req.phase = Phase.QUEUED
         self.queue.append(req)
 

@@ -10,8 +10,9 @@ the model file (reference: qwen3_runtime/utils/loader.py:33-54).
 from __future__ import annotations
 
 from ..config.model import Qwen3Config
+from ..config.presets import PRESET_PAGE_SIZE, PRESETS
 from ..parts.plan import CacheSpec, LayerSpec, ModelPlan, PartSpec, RunStep
-from ..registry import register_architecture
+from ..registry import register_architecture, register_preset
 
 
 def plan_qwen3(cfg: Qwen3Config) -> ModelPlan:
@@ -80,3 +81,5 @@ def _rmsnorm(cfg: Qwen3Config, name: str) -> PartSpec:
 
 
 register_architecture(Qwen3Config.architecture, Qwen3Config.from_dict, plan_qwen3)
+for _name, _cfg in PRESETS.items():
+    register_preset(_name, _cfg.to_dict(), PRESET_PAGE_SIZE.get(_name, 16))

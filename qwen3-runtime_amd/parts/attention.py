@@ -78,6 +78,15 @@ class GroupedQueryAttention(Mixer):
             self.q_norm = fetch.vector_f32(self._name("q_norm"))
             self.k_norm = fetch.vector_f32(self._name("k_norm"))
 
+    def step_cost(self, spans, rows, elem_bytes):
+        cost = super().step_cost(spans, rows, elem_bytes)  # the four projections
+        for q, kv in spans:  # scores and weighted values: 4 D operations per (query head, visible key)
+            first = kv - q
+            pairs = sum(min(first + i + 1, self.window or kv) for i in range(q)) if self.window else \
+                q * first + q * (q + 1) // 2
+            cost.flop += 4.0 * self.num_heads * self.head_dim * pairs
+        return cost
+
     def forward(self, ctx, x, cache):
         ops = ctx.ops
         nq, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim

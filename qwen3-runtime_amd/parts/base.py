@@ -46,6 +46,25 @@ class WeightFetcher(Protocol):
     def constant(self, tensor: torch.Tensor) -> torch.Tensor: ...
 
 
+@dataclass
+class StepCost:
+    """What a step asks of the device, for rooflines: bytes of each tensor it reads (by file
+    name: a tensor two parts share, or a layer that runs twice, is read once) and
+    floating-point operations."""
+
+    weight_bytes: dict[str, int] = field(default_factory=dict)
+    flop: float = 0.0
+
+    def add(self, other: "StepCost") -> None:
+        for name, n in other.weight_bytes.items():
+            self.weight_bytes[name] = max(self.weight_bytes.get(name, 0), n)
+        self.flop += other.flop
+
+    @property
+    def total_weight_bytes(self) -> int:
+        return sum(self.weight_bytes.values())
+
+
 class Part:
     """Base of all parts: holds the tensor-name map, declares and loads tensors."""
 
@@ -69,6 +88,23 @@ class Part:
 
     def children(self) -> Sequence["Part"]:
         return ()
+
+    def step_cost(self, spans: Sequence[tuple[int, int]], rows: int, elem_bytes: int) -> StepCost:
+        """Bytes and operations of one run of this part (children not included) over a step whose
+        sequences are ``spans`` = (tokens of the step, tokens in the cache after it), with logits
+        wanted at ``rows`` places. The default fits a part whose tensors are all read whole and
+        whose matrices each multiply every token once; a part for which that is wrong (a table
+        that is only looked up, experts of which few run, attention's own products) says so."""
+        tokens = sum(q for q, _ in spans)
+        cost = StepCost()
+        for decl in self.tensor_decls():
+            n = 1
+            for dim in decl.shape:
+                n *= dim
+            cost.weight_bytes[decl.file_name] = n * elem_bytes
+            if decl.init == "matrix" and len(decl.shape) == 2:
+                cost.flop += 2.0 * tokens * n
+        return cost
 
     def _name(self, logical: str) -> str:
         try:
@@ -135,11 +171,14 @@ class CacheView:
     spec: CacheSpec
     writes: bool = True
     group: GroupView | None = None
-    # paged_kv: keys [pages, heads, page_size, D]; values [pages, heads, D, page_size]
+    # paged_kv: keys [pages, heads, page_size, D]; values [pages, heads, Dv, page_size]
     k: torch.Tensor | None = None
     v: torch.Tensor | None = None
     # state: [slots, *shape]
     state: torch.Tensor | None = None
+    # any paged cache: stream name -> [pages, *PagedStream.page_shape(page_size)]; for
+    # "paged_kv" the entries "k" and "v" are the tensors above
+    pages: dict[str, torch.Tensor] = field(default_factory=dict)
 
 
 @dataclass

@@ -9,7 +9,7 @@ The embedding starts the float32 residual stream; logits come out in float32.
 from __future__ import annotations
 
 from ..registry import register_part
-from .base import Part
+from .base import Part, StepCost
 from .plan import TensorDecl
 
 
@@ -32,6 +32,11 @@ class TokenEmbedding(Part):
     def forward(self, ctx, ids):
         return ctx.ops.embed(ids, self.weight)
 
+    def step_cost(self, spans, rows, elem_bytes):
+        # a lookup: one row of the table per token, no arithmetic
+        tokens = sum(q for q, _ in spans)
+        return StepCost({self._name("weight"): min(tokens, self.vocab_size) * self.hidden_size * elem_bytes}, 0.0)
+
 
 @register_part("head", "linear_head")
 class LinearHead(Part):
@@ -53,3 +58,8 @@ class LinearHead(Part):
 
     def forward(self, ctx, x):
         return ctx.ops.linear(x, self.weight, out_f32=True)
+
+    def step_cost(self, spans, rows, elem_bytes):
+        # the whole matrix, multiplied with the wanted rows only
+        n = self.vocab_size * self.hidden_size
+        return StepCost({self._name("weight"): n * elem_bytes}, 2.0 * rows * n)

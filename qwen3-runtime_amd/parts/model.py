@@ -11,7 +11,7 @@ import math
 from typing import Sequence
 
 from ..registry import part_class
-from .base import CacheView, Part, StepContext
+from .base import CacheView, Part, StepContext, StepCost
 from .plan import ModelPlan, PartSpec, TensorDecl
 
 
@@ -74,6 +74,16 @@ class DecoderModel:
     def portion_multiple(self) -> int:
         """Least common multiple of what the parts ask of a prompt's portions."""
         return math.lcm(*(max(1, int(part.portion_multiple)) for part in self.parts()))
+
+    def step_cost(self, spans, rows: int, elem_bytes: int) -> StepCost:
+        """Bytes of weights and floating-point operations of one step (``Part.step_cost``), summed
+        over the parts in the order they run: a layer named twice computes twice and is read once."""
+        cost = StepCost()
+        runs = [self.embedding] + [self.blocks[step.layer] for step in self.plan.order] + [self.final_norm, self.head]
+        for top in runs:
+            for part in walk(top):
+                cost.add(part.step_cost(spans, rows, elem_bytes))
+        return cost
 
     def tensor_decls(self) -> list[TensorDecl]:
         """Every tensor the model reads, once per file name."""

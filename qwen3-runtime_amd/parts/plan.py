@@ -46,13 +46,36 @@ class TensorDecl:
 
 
 @dataclass(frozen=True)
+class PagedStream:
+    """One tensor a paged cache keeps for every token: ``heads`` x ``width`` elements.
+
+    Within a page the tensor is ``[head, offset, width]``, or, ``transposed``,
+    ``[head, width, offset]`` (the tokens of a page contiguous for one element: what a kernel
+    wants that multiplies probabilities over keys with values)."""
+
+    name: str
+    heads: int
+    width: int
+    transposed: bool = False
+
+    def page_shape(self, page_size: int) -> tuple[int, int, int]:
+        return (self.heads, self.width, page_size) if self.transposed else (self.heads, page_size, self.width)
+
+    def elements_per_token(self) -> int:
+        return self.heads * self.width
+
+
+@dataclass(frozen=True)
 class CacheSpec:
     """What one cache owner keeps between steps.
 
     ``kind == "paged_kv"``: keys and values for every token (or the last
-    ``window`` tokens), ``heads`` x ``head_dim`` each, held in pages.
-    ``kind == "state"``: a fixed-size tensor of ``shape`` per request, held in a
-    slot; ``dtype`` is a torch dtype name or ``"model"`` for the model's dtype.
+    ``window`` tokens), ``heads`` x ``head_dim`` keys and ``heads`` x ``value_dim``
+    values (``head_dim`` when None), held in pages; the values transposed within a
+    page. ``kind == "paged"``: any other set of per-token tensors, named by
+    ``streams`` (one latent vector per token, say), with the same pages, tables and
+    window. ``kind == "state"``: a fixed-size tensor of ``shape`` per request, held
+    in a slot; ``dtype`` is a torch dtype name or ``"model"`` for the model's dtype.
     """
 
     kind: str
@@ -61,11 +84,32 @@ class CacheSpec:
     window: int | None = None
     shape: tuple[int, ...] = ()
     dtype: str = "model"
+    value_dim: int | None = None
+    streams: tuple[PagedStream, ...] = ()
+
+    @property
+    def paged(self) -> bool:
+        return self.kind in ("paged_kv", "paged")
+
+    def page_streams(self) -> tuple[PagedStream, ...]:
+        """The per-token tensors of a paged cache; a ``CacheView`` holds one device tensor for each,
+        under the stream's name."""
+        if self.kind == "paged_kv":
+            return (PagedStream("k", self.heads, self.head_dim),
+                    PagedStream("v", self.heads, self.head_dim if self.value_dim is None else self.value_dim, True))
+        if self.kind == "paged":
+            if not self.streams:
+                raise ValueError("a cache of kind 'paged' names its streams")
+            return tuple(self.streams)
+        return ()
+
+    def elements_per_token(self) -> int:
+        return sum(s.elements_per_token() for s in self.page_streams())
 
     def group_key(self) -> tuple:
         """Caches with equal keys share pages' geometry and lifetime, hence a pool."""
-        if self.kind == "paged_kv":
-            return ("paged_kv", self.heads, self.head_dim, self.window)
+        if self.paged:
+            return ("paged", self.page_streams(), self.window)
         return ("state", tuple(self.shape), self.dtype)
 
 

@@ -27,6 +27,8 @@ class Architecture:
 
 _ARCHITECTURES: dict[str, Architecture] = {}
 _PARTS: dict[str, dict[str, type]] = {role: {} for role in ROLES}
+# named configurations: name -> (config.json as a dict, page size it is run with by default)
+_PRESETS: dict[str, tuple[dict, int]] = {}
 
 
 def register_architecture(name: str, read_config, make_plan) -> Architecture:
@@ -56,6 +58,42 @@ def architecture_for(raw_config: Mapping[str, Any]) -> Architecture:
     raise ValueError(
         f"no registered architecture among {list(names)}; registered: {sorted(_ARCHITECTURES)}"
     )
+
+
+def register_preset(name: str, raw_config: Mapping[str, Any], page_size: int = 16) -> None:
+    """A named configuration (a config.json as a dict, ``architectures`` included) that the
+    entry points build with random weights: ``--preset NAME`` on the command line, and the
+    model ``LLM(None)`` makes is the first one registered."""
+    if not raw_config.get("architectures"):
+        raise ValueError(f"preset {name!r}: the configuration names no architecture")
+    _PRESETS[name] = (dict(raw_config), int(page_size))
+
+
+def unregister_preset(name: str) -> None:
+    _PRESETS.pop(name, None)
+
+
+def preset_names() -> list[str]:
+    _load_builtin()
+    return list(_PRESETS)
+
+
+def preset_config(name: str | None = None) -> dict:
+    """The configuration registered under ``name`` (None: the first registered), as a fresh dict."""
+    _load_builtin()
+    if name is None:
+        if not _PRESETS:
+            raise ValueError("no preset is registered")
+        name = next(iter(_PRESETS))
+    try:
+        return dict(_PRESETS[name][0])
+    except KeyError:
+        raise ValueError(f"unknown preset {name!r}; presets: {list(_PRESETS)}") from None
+
+
+def preset_page_size(name: str) -> int:
+    _load_builtin()
+    return _PRESETS[name][1] if name in _PRESETS else 16
 
 
 def register_part(role: str, kind: str, cls: type | None = None):

@@ -28,11 +28,15 @@ MAX_LIVE = 4
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
-    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--model", default=None, help="folder with config.json and model.safetensors")
+    ap.add_argument("--preset", default=None,
+                    help="instead of --model: seeded random weights of a registered configuration")
+    ap.add_argument("--seed", type=int, default=0, help="seed of --preset's weights")
     ap.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
-    ap.add_argument("--max-tokens", type=int, required=True,
+    ap.add_argument("--max-tokens", type=int, default=None,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
+    ap.add_argument("--num-pages", type=int, default=None, help="instead of --max-tokens: pages per cache group")
     ap.add_argument("--page-size", type=int, default=16)
     args = ap.parse_args(argv)
 
@@ -46,12 +50,28 @@ def main(argv=None) -> int:
         ap.error(f"--page-size must divide {CAPACITY_UNIT}")
     out = Path(args.out)
     out.mkdir(parents=True, exist_ok=True)
-    num_pages = max(1, -(-args.max_tokens // CAPACITY_UNIT)) * (CAPACITY_UNIT // args.page_size)
+    if (args.model is None) == (args.preset is None):
+        ap.error("give --model DIR or --preset NAME")
+    if (args.max_tokens is None) == (args.num_pages is None):
+        ap.error("give --max-tokens N or --num-pages N")
+    if args.num_pages is not None:
+        num_pages = args.num_pages
+    else:
+        num_pages = max(1, -(-args.max_tokens // CAPACITY_UNIT)) * (CAPACITY_UNIT // args.page_size)
     engine = EngineConfig(page_size=args.page_size, num_pages=num_pages, max_num_seqs=MAX_LIVE,
                           dtype=args.dtype, device="cuda:0", hip_graph=False)
-    print(f"[trace_run] loading {args.model} ({args.dtype}, {num_pages} pages of {args.page_size})",
+    print(f"[trace_run] loading {args.model or args.preset} ({args.dtype}, {num_pages} pages of {args.page_size})",
           file=sys.stderr, flush=True)
-    loaded = load(args.model, engine)
+    if args.preset is not None:
+        from .engine.factory import build_model
+        from .registry import preset_config
+        from .weights import RandomSource
+
+        raw = preset_config(args.preset)
+        source = RandomSource(build_model(raw)[1].tensor_decls(), args.seed, norm_jitter=0.1)
+        loaded = load(None, engine, source=source, raw_config=raw)
+    else:
+        loaded = load(args.model, engine)
     runner, cache = loaded.runner, loaded.cache
 
     for line in sys.stdin:

@@ -288,3 +288,44 @@ def test_random_lifetimes_keep_every_page_accounted_for(seed, num_pages, page_si
     m.check()
     assert all(g.pool.num_free == num_pages for g in m.groups)
     assert m.slots.num_free == 5
+
+
+# --- what a paged cache holds per token is the spec's to say ---------------------------------------
+def test_streams_of_a_paged_cache_decide_storage_views_and_bytes():
+    from qwen3_runtime_amd.parts.base import GroupView
+    from qwen3_runtime_amd.parts.plan import PagedStream
+
+    kv = CacheSpec("paged_kv", heads=2, head_dim=16, value_dim=24)          # values wider than keys
+    latent = CacheSpec("paged", streams=(PagedStream("latent", 1, 40), PagedStream("rope_key", 1, 8, True)))
+    assert kv.group_key() != FULL.group_key() and latent.group_key() != kv.group_key()
+    # bytes: 2 * (16 + 24) elements per token for the first, 40 + 8 for the second
+    assert CacheManager.bytes_per_page([kv, latent, FULL], 8, 2) == 8 * 2 * (80 + 48 + 64)
+    m = manager(5, 8, [kv, latent, kv], allocate=True)
+    assert len(m.groups) == 2
+    views = [GroupView(8, None, None, None)] * 2
+    a, b, c = (m.view(i, views) for i in range(3))
+    assert a.k.shape == (5, 2, 8, 16) and a.v.shape == (5, 2, 24, 8) and a.pages["v"] is a.v
+    assert b.k is None and b.pages["latent"].shape == (5, 1, 8, 40) and b.pages["rope_key"].shape == (5, 1, 8, 8)
+    # two caches of one group have storage of their own
+    a.k.fill_(1.0)
+    assert float(c.k.abs().sum()) == 0.0 and c.k.shape == a.k.shape
+    with pytest.raises(ValueError, match="names its streams"):
+        CacheSpec("paged").page_streams()
+
+
+def test_bytes_a_step_reads_follow_windows_and_states():
+    specs = [FULL, CacheSpec("paged_kv", heads=1, head_dim=8, window=6), CacheSpec("state", shape=(5,), dtype="float32")]
+    m = manager(8, 4, specs, allocate=True)
+    # all keys and values of the full cache, at most six tokens of the windowed one, the state once per request
+    assert m.bytes_read([10, 3], dtype_bytes=2) == (13 * 64 + (6 + 3) * 16) * 2 + 2 * 5 * 4
+
+
+def test_a_window_group_needs_its_windows_pages_only():
+    window = CacheSpec("paged_kv", heads=1, head_dim=8, window=6)
+    m = manager(3, 4, [window])
+    assert m.can_ever_hold(10_000) == (True, "")         # six positions touch at most three pages of four
+    ok, why = manager(2, 4, [window]).can_ever_hold(100)
+    assert not ok and "window 6" in why and "needs 3" in why
+    assert manager(2, 4, [window]).can_ever_hold(8)[0]    # a short request needs its own length only
+    ok, why = manager(3, 4, [window, FULL]).can_ever_hold(13)
+    assert not ok and "needs 4 cache pages" in why        # the group that keeps every key decides

@@ -462,3 +462,165 @@ def test_toy_architecture_generates_through_the_engine_in_portions_it_asked_for(
         for _ in range(5):
             ids.append(int(toy_plain(toy_folder, ids)[-1].argmax()))
         assert out == ids[len(p):]
+
+
+def test_toy_architecture_from_its_configuration_alone(toy_folder):
+    """``build_engine(None, config=...)`` with the toy's config.json as a dict (no folder, no typed
+    configuration class, no preset): seeded random weights on the device, generation through
+    scheduler and sampler, and what a measurement needs (bytes a step reads, its operations) from
+    the parts and the cache manager, with no edit in the package."""
+    from qwen3_runtime_amd.llm import build_engine
+    from qwen3_runtime_amd.weights import RandomSource
+
+    eng = build_engine(None, config=TOY, seed=5, norm_jitter=0.1, block_size=8, num_kv_blocks=24, max_num_seqs=2,
+                       max_num_batched_tokens=32, dtype="float32", device=DEV)
+    prompts = list(traces.make_requests(TOY["vocab_size"], [21, 6], seed=9).values())
+    outs = eng.generate_batch(prompts, max_tokens=4)
+    # the same weights, written to a folder, through the plain computation
+    model = eng.loaded.model
+    src = RandomSource(model.tensor_decls(), 5, norm_jitter=0.1)
+    import json
+    import tempfile
+
+    from safetensors.torch import save_file
+
+    with tempfile.TemporaryDirectory() as folder:
+        save_file({d.file_name: src.get(d.file_name).contiguous() for d in model.tensor_decls()},
+                  f"{folder}/model.safetensors")
+        Path(folder, "config.json").write_text(json.dumps(TOY))
+        for p, out in zip(prompts, outs):
+            ids = list(p)
+            for _ in range(4):
+                ids.append(int(toy_plain(folder, ids)[-1].argmax()))
+            assert out == ids[len(p):]
+    # a decode step of two requests that hold 30 and 9 tokens
+    spans = [(1, 30), (1, 9)]
+    cost = model.step_cost(spans, rows=2, elem_bytes=4)
+    h, d, v, inter = TOY["hidden_size"], TOY["head_dim"], TOY["vocab_size"], TOY["intermediate_size"]
+    attn0 = (4 + 2 + 2) * d * h + h * 4 * d
+    attn2 = (2 + 1 + 1) * d * h + h * 2 * d
+    ff = 3 * h * inter
+    experts = TOY["experts"] * (h + 3 * h * TOY["expert_size"])
+    # layers 0 and 2 run twice: their matrices are read once and multiply twice; the embedding is
+    # looked up (two rows), the head multiplies the two wanted rows
+    want_flop = 2 * 2 * (2 * (attn0 + ff) + 2 * (attn2 + ff) + experts) + 2 * 2 * v * h
+    want_flop += 4 * d * (2 * 4 * (30 + 9) + 2 * 2 * (min(30, TOY["window"]) + min(9, TOY["window"])))
+    assert cost.flop == pytest.approx(want_flop)
+    norms = 4 * (6 * h + 4 * d + h) + 4 * h          # norm vectors, q/k norms, the toy mixer's gain, final norm
+    assert cost.total_weight_bytes == 4 * (attn0 + attn2 + 2 * ff + experts + v * h + 2 * h) + norms
+    # the cache: two full groups' worth of keys and values, a window, one state per request
+    read = eng.cache.bytes_read([30, 9], 4)
+    assert read == 4 * (2 * (2 * 2 * d) * 39 + (2 * 1 * d) * (11 + 9)) + 2 * h * 4
+
+
+# ------------------------------------------------------------------------------------------------
+# A mixer whose paged cache is neither keys nor values: one latent vector per token.
+# ------------------------------------------------------------------------------------------------
+LATENT = {"architectures": ["ToyLatentForCausalLM"], "vocab_size": 90, "hidden_size": 32, "latent": 12,
+          "intermediate_size": 48, "eps": 1e-5, "max_positions": 256}
+
+
+@pytest.fixture(scope="module")
+def latent_folder(tmp_path_factory):
+    from qwen3_runtime_amd.parts.base import Mixer
+    from qwen3_runtime_amd.parts.plan import (CacheSpec, LayerSpec, ModelPlan, PagedStream, PartSpec, RunStep,
+                                              TensorDecl)
+    from qwen3_runtime_amd.registry import (register_architecture, register_part, unregister_architecture,
+                                            unregister_part)
+    from qwen3_runtime_amd.weights import write_model_folder
+
+    @register_part("mixer", "toy_latent")
+    class LatentMixer(Mixer):
+        """c_t = W_in x_t is stored per token in pages of its own (one stream, no keys, no values);
+        y_t = W_out mean(c_0 .. c_t). It gathers with torch on the host's say-so, so no graph."""
+
+        graph_capturable = False
+
+        def __init__(self, hidden_size, latent, tensors=None):
+            super().__init__(tensors)
+            self.h, self.r = hidden_size, latent
+
+        def cache_spec(self):
+            return CacheSpec("paged", streams=(PagedStream("latent", 1, self.r),))
+
+        def tensor_decls(self):
+            return [TensorDecl(self._name("in"), (self.r, self.h)), TensorDecl(self._name("out"), (self.h, self.r))]
+
+        def load(self, fetch):
+            self.w_in, self.w_out = fetch.matrix(self._name("in")), fetch.matrix(self._name("out"))
+
+        def forward(self, ctx, x, cache):
+            latent = ctx.ops.linear(x, self.w_in)
+            pages = cache.pages["latent"]                         # [pages, 1, page_size, r]
+            ps = cache.group.page_size
+            flat = pages.view(-1, self.r)
+            flat.index_copy_(0, cache.group.slots.long(), latent.to(flat.dtype))
+            mean = torch.empty((ctx.num_tokens, self.r), dtype=torch.float32, device=x.device)
+            row = 0
+            for s, (q, kv) in enumerate(zip(ctx.q_lens_host, ctx.kv_lens_host)):
+                pos = torch.arange(kv, device=x.device)
+                places = cache.group.block_table[s, pos // ps].long() * ps + pos % ps
+                sums = flat[places].float().cumsum(0)
+                mean[row: row + q] = sums[kv - q:] / (pos[kv - q:] + 1)[:, None]
+                row += q
+            return ctx.ops.linear(mean.to(x.dtype), self.w_out)
+
+    def make_plan(c):
+        h = c["hidden_size"]
+        norm = lambda name: PartSpec("rmsnorm", {"size": h, "eps": c["eps"]}, {"weight": name})
+        layers, caches, order = [], [], []
+        for i in range(2):
+            mixer = PartSpec("toy_latent", {"hidden_size": h, "latent": c["latent"]},
+                             {"in": f"lat.{i}.in", "out": f"lat.{i}.out"})
+            ff = PartSpec("swiglu", {"hidden_size": h, "intermediate_size": c["intermediate_size"]},
+                          {k: f"lat.{i}.ff.{k}" for k in ("gate", "up", "down")})
+            layers.append(LayerSpec(PartSpec("pre_norm"), mixer, ff,
+                                    {"input": norm(f"lat.{i}.norm_in"), "post_mixer": norm(f"lat.{i}.norm_post")}))
+            caches.append(CacheSpec("paged", streams=(PagedStream("latent", 1, c["latent"]),)))
+            order.append(RunStep(i, i))
+        sizes = {"vocab_size": c["vocab_size"], "hidden_size": h}
+        return ModelPlan(h, c["vocab_size"], c["max_positions"],
+                         PartSpec("token_embedding", sizes, {"weight": "lat.embed"}), layers, caches, order,
+                         norm("lat.norm"), PartSpec("linear_head", sizes, {"weight": "lat.embed"}))
+
+    register_architecture("ToyLatentForCausalLM", dict, make_plan)
+    folder = write_model_folder(tmp_path_factory.mktemp("latent"), LATENT, seed=3)
+    yield folder
+    unregister_architecture("ToyLatentForCausalLM")
+    unregister_part("mixer", "toy_latent")
+
+
+def latent_plain(folder, ids):
+    c, w = P.read_model(folder)
+    x = w["lat.embed"][torch.as_tensor(ids)]
+    steps = torch.arange(1, len(ids) + 1).double()[:, None]
+    for i in range(2):
+        n = P.rms_norm(x, w[f"lat.{i}.norm_in"], c["eps"])
+        x = x + ((n @ w[f"lat.{i}.in"].T).cumsum(0) / steps) @ w[f"lat.{i}.out"].T
+        n = P.rms_norm(x, w[f"lat.{i}.norm_post"], c["eps"])
+        x = x + P.feed_forward(n, {f"f.{k}_proj.weight": w[f"lat.{i}.ff.{k}"] for k in ("gate", "up", "down")}, "f")
+    return P.rms_norm(x, w["lat.norm"], c["eps"]) @ w["lat.embed"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_paged_cache_of_latent_vectors(latent_folder, dtype):
+    """The cache manager pages whatever per-token tensors a mixer's ``CacheSpec`` names: block
+    tables, slots, reuse of pages and the step function are those of keys and values. Mixed
+    steps in a pool at its peak, against the whole-sequence computation."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    reqs = traces.make_requests(LATENT["vocab_size"], [30, 7, 52, 18, 41, 9], seed=2)
+    steps = traces.mixed(reqs, seed=1, max_live=3)
+    page = 8
+    pages = traces.peak_tokens(steps, unit=page) // page
+    assert pages < sum(-(-len(t) // page) for t in reqs.values())
+    loaded = load(latent_folder, EngineConfig(page_size=page, num_pages=pages, max_num_seqs=3, dtype=dtype, device=DEV))
+    assert not loaded.runner.hip_graph and loaded.runner.repeatable
+    assert loaded.cache.bytes_per_page(loaded.model.plan.caches, page, 2) == 2 * 12 * page * 2
+    got = traces.replay(loaded, steps, poison_freed=True)
+    want = {(rid, p): row.float() for rid, toks in reqs.items() for p, row in enumerate(latent_plain(latent_folder, toks))}
+    if dtype == "float32":
+        traces.compare(got, want, atol=5e-5, rtol=5e-5)
+    else:
+        traces.compare_rounding_noise(got, want)

@@ -242,3 +242,30 @@ def test_sampling_params_validation():
     assert SamplingParams().is_greedy() and SamplingParams(temperature=-1.0).is_greedy()
     assert not SamplingParams(temperature=0.5).is_greedy()
     assert SamplingParams(presence_penalty=0.1).has_penalties() and not SamplingParams().has_penalties()
+
+
+def test_a_windowed_model_serves_requests_longer_than_its_pool():
+    """One group of caches with a window of 12 tokens and a pool of five pages of four: a request of
+    200 tokens is admitted (its window's pages are all it ever needs at once), its prompt is cut to
+    what the pool holds, pages behind the window come back as it goes, and it ends."""
+    cfg = EngineConfig(page_size=4, num_pages=5, max_num_seqs=2, max_num_batched_tokens=64, dtype="float32",
+                       device="cpu")
+    cache = CacheManager([CacheSpec("paged_kv", heads=1, head_dim=8, window=12)], page_size=4, num_pages=5,
+                         max_requests=4, device="cpu", dtype=torch.float32, allocate=False)
+    s = Scheduler(cfg, cache, 100_000)
+    req = Request(list(range(150)), max_tokens=50)
+    s.add(req)
+    grants = []
+    while not s.is_finished():
+        batch = s.schedule()
+        assert batch == [req] and 1 <= req.grant <= 20
+        grants.append(req.grant)
+        caught_up = cache.length(req.request_id) + req.grant >= len(req.token_ids)
+        run(s, batch, [7 if caught_up else None])
+        cache.check()
+        assert len(grants) < 400
+    assert req.finish_reason == "length" and len(req.output_tokens) == 50
+    assert max(grants) > 1 and cache.num_free_pages == 5
+    # a model that keeps every key refuses the same request in the same pool
+    with pytest.raises(RuntimeError, match="needs 50 cache pages"):
+        scheduler(num_pages=5, page_size=4).add(Request(list(range(150)), max_tokens=50))

@@ -150,8 +150,8 @@ def replay(loaded, steps, check_cache=True, page_users=None, poison_freed=False)
     out = {}
 
     def poison(group, pages):
-        group.storage[:, 0, pages] = float("nan")
-        group.storage[:, 1, pages] = float("inf")
+        for i, store in enumerate(group.storage):  # keys, values (or whatever streams the cache has)
+            store[:, pages] = float("nan") if i % 2 == 0 else float("inf")
 
     if poison_freed:
         for g in cache.groups:
@@ -183,7 +183,7 @@ def replay(loaded, steps, check_cache=True, page_users=None, poison_freed=False)
             cache.release(rid)
             if poison_freed:
                 for g, pages in zip(cache.groups, held):
-                    poison(g, torch.tensor(pages, dtype=torch.long, device=g.storage.device))
+                    poison(g, torch.tensor(pages, dtype=torch.long, device=g.storage[0].device))
         if check_cache:
             cache.check()
     assert not cache.live_requests()
@@ -237,6 +237,38 @@ def compare_rounding_noise(got, want, rms_bound=0.015, worst_bound=0.08):
     assert rms < rms_bound * std, f"rms error {rms:.4f} against a logit deviation of {std:.3f}"
     MEASURED_NOISE.append((rms / std, worst / std, os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0]))
     return rms / std, worst / std
+
+
+def plain_logprobs(cfg, weights, prompt, tokens):
+    """The plain implementation's log-probability of each of ``tokens`` following ``prompt`` (and
+    each other), how far each lies below the best token of its place, and the logits' deviation."""
+    from plain import qwen3_plain as P
+
+    logits = P.forward(cfg, weights, list(prompt) + list(tokens))[len(prompt) - 1: -1].double()
+    picked = logits[range(len(tokens)), list(tokens)]
+    logprobs = torch.log_softmax(logits, dim=-1)[range(len(tokens)), list(tokens)]
+    return logprobs.tolist(), (logits.max(dim=-1).values - picked).tolist(), float(logits.std())
+
+
+def compare_logprobs(got, want, std, rms_bound=0.015, worst_bound=0.08):
+    """Log-probabilities of given tokens, engine against plain (or graph against eager), by the
+    measure of ``compare_rounding_noise``: in units of the logits' deviation ``std``."""
+    err = torch.tensor(got, dtype=torch.float64) - torch.tensor(want, dtype=torch.float64)
+    assert err.numel() and err.numel() == len(want)
+    rms, worst = float(err.pow(2).mean().sqrt()), float(err.abs().max())
+    assert worst < worst_bound * std, f"largest log-probability error {worst:.4f} at token {int(err.abs().argmax())}; logit deviation {std:.3f}"
+    assert rms < rms_bound * std, f"rms log-probability error {rms:.4f} against a logit deviation of {std:.3f}"
+    MEASURED_NOISE.append((rms / std, worst / std, os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0]))
+
+
+def check_tokens_chosen_in_bfloat16(cfg, weights, prompt, tokens, bound=0.08):
+    """Tokens an engine chose greedily in bfloat16, judged by the plain implementation given the
+    same context: each is the plain model's best token or lies below it by less than the
+    rounding noise of two logits (``bound`` of the logits' deviation). A wrong cache or mask
+    picks tokens far below the best."""
+    _, below_best, std = plain_logprobs(cfg, weights, prompt, tokens)
+    worst = max(below_best)
+    assert worst < bound * std, f"token {below_best.index(worst)} lies {worst:.4f} below the plain model's best; deviation {std:.3f}"
 
 
 def compare(got, want, atol, rtol):
