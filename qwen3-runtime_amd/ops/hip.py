@@ -285,7 +285,7 @@ class HipOps:
             c_int(m), c_int(n), c_int(k), c_int(0), c_int(kernel), c_int(1), _stream()))
         return out
 
-    # rows from which a library product is tried in two column chunks
+    # rows from which a library product is made in two column chunks; False: never
     library_split_min_rows = 256
 
     def _library_product(self, x, w):
@@ -293,14 +293,16 @@ class HipOps:
 
         The library's kernels work on tiles of the result (256 x 256 for these shapes), and a
         result whose tiles do not fill the 256 compute units a whole number of times leaves
-        them idle in the last round: 2,048 x 19,456 is 608 tiles, 2.4 rounds. A first chunk of
-        columns that fills whole rounds and a second call for the rest took 175 us instead of
-        210 there, and 293 instead of 393 at 4,096 rows. Whether it pays depends on the
-        library's own choices, so each shape (rows in units of 256, N, K) is timed both ways
-        the first time it is met, outside stream capture, and the faster way is kept."""
+        them idle in the last round: 2,048 x 19,456 is 608 tiles, 2.4 rounds (0.93 PFLOP/s, where
+        2,048 x 24,576, three whole rounds, runs at 1.45). A first chunk of columns that fills
+        whole rounds and a second call for the rest is faster wherever such a cut exists: over the
+        products of the 1.7B to 32B sizes at 256 to 8,192 rows the two calls took 0.69 to 0.99 of
+        the one call's time (0.80 for the case above), 1.02 at worst. The cut depends on the
+        shape alone, so equal inputs give equal bits in every process (the two ways use other
+        library kernels, which round differently)."""
         m, k = x.shape
         n = w.shape[0]
-        split = self._library_split(x, w)
+        split = self.library_split(m, n)
         if not split:
             return torch.matmul(x, w.t())
         out = torch.empty((m, n), dtype=x.dtype, device=x.device)
@@ -308,42 +310,15 @@ class HipOps:
         torch.mm(x, w[split:].t(), out=out[:, split:])
         return out
 
-    def _library_split(self, x, w) -> int:
-        m, k = x.shape
-        n = w.shape[0]
-        if m < self.library_split_min_rows:
+    def library_split(self, m: int, n: int) -> int:
+        """Columns of the first chunk (0: one call): the most whose 256 x 256 tiles fill the
+        compute units a whole number of times, if that leaves a second chunk."""
+        if not self.library_split_min_rows or m < self.library_split_min_rows:
             return 0
         row_tiles = -(-m // 256)
         per_round = 256 * max(1, 256 // row_tiles)  # columns whose tiles fill the compute units once
         split = (n // per_round) * per_round
-        if not 0 < split < n:
-            return 0
-        plans = self.__dict__.setdefault("_library_plans", {})
-        key = (row_tiles, n, k)
-        if key not in plans:
-            if torch.cuda.is_current_stream_capturing():
-                return 0  # not timed yet, and no timing inside a capture
-            out = torch.empty((m, n), dtype=x.dtype, device=x.device)
-
-            def whole():
-                torch.mm(x, w.t(), out=out)
-
-            def chunked():
-                torch.mm(x, w[:split].t(), out=out[:, :split])
-                torch.mm(x, w[split:].t(), out=out[:, split:])
-
-            def timed(fn):
-                fn()
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                for _ in range(3):
-                    fn()
-                b.record()
-                b.synchronize()
-                return a.elapsed_time(b)
-
-            plans[key] = split if timed(chunked) < 0.97 * timed(whole) else 0
-        return plans[key]
+        return split if 0 < split < n else 0
 
     def _own_kernel(self, m: int, k: int, tiled, form: str) -> int | None:
         """Which of the library's kernels multiplies ``m`` rows by this weight: 0 the few-row

@@ -35,7 +35,7 @@ def test_bench_line_has_the_contract_fields():
         assert key in rec, key
     assert rec["n_gpus"] == 1 and rec["steps"] == 8 and rec["warmup"] == 2 and rec["higher_is_better"] is True
     assert len(rec["config"]) <= 20 and all(not isinstance(v, (dict, list)) for v in rec["config"].values())
-    assert rec["config"]["layers"] == 2 and rec["config"]["layers_of_full_model"] == 36
+    assert rec["config"]["num_hidden_layers"] == 2 and rec["config"]["layers_of_full_model"] == 36
     assert {"value", "tokens", "ms", "frac"} <= set(rec["prefill"]) and rec["prefill"]["tokens"] == 2048
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0
     assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / rec["roofline"]["peak"]) < 1e-3
@@ -43,10 +43,12 @@ def test_bench_line_has_the_contract_fields():
     assert all(isinstance(v, float) for v in rec["points"].values())
     assert abs(rec["value"] - 8 * 1000.0 / rec["ms_per_step"]) / rec["value"] < 0.01
 
-    # the arithmetic behind the fractions, recomputed here from the sizes the line names
+    # the arithmetic behind the fractions (which bench.py takes from the model's parts and the cache
+    # manager), recomputed here from the sizes the line names, with the architecture's own formulas
     c = rec["config"]
-    h, d, i, v, layers = c["hidden"], c["head_dim"], c["intermediate"], c["vocab"], c["layers"]
-    q, kv = c["heads"] * d, c["kv_heads"] * d
+    h, d, i, v, layers = c["hidden_size"], c["head_dim"], c["intermediate_size"], c["vocab_size"], c["num_hidden_layers"]
+    q, kv = c["num_attention_heads"] * d, c["num_key_value_heads"] * d
+    assert c["tie_word_embeddings"] is True
     per_layer = h * (q + 2 * kv) + q * h + 3 * h * i + 2 * h + 2 * d       # matrices, two norms, q/k norms
     weight_bytes = 2 * (v * h + layers * per_layer + h)                    # tied table once, final norm
     kv_per_token = 2 * layers * kv * 2

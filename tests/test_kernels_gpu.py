@@ -259,23 +259,26 @@ def test_gemm_bf16_large_uses_blas_and_agrees(ops):
 
 def test_library_product_in_two_column_chunks():
     """Products with many rows go to the vendor library, whole or as two calls over column chunks
-    of one result tensor, whichever was faster when the shape was first met. Both ways, and the
-    way chosen, give the float64 product."""
+    of one result tensor; which, follows from the shape alone, so two processes give the same
+    bits. Both ways give the float64 product."""
     from qwen3_runtime_amd.ops.hip import HipOps
 
     ops = HipOps()
     m, n, k = 300, 33000, 64                       # two row tiles: 32,768 columns fill the chip once
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.05)
     want = x.double() @ w.double().T
-    close(ops.linear(x, w), want, 3e-2, 3e-2)      # timed both ways now, one of them kept
-    assert ops._library_plans[(2, n, k)] in (0, 32768)
-    for split in (0, 32768):
-        ops._library_plans[(2, n, k)] = split
-        got = ops.linear(x, w)
-        assert got.is_contiguous() and got.shape == (m, n)
-        close(got, want, 3e-2, 3e-2)
-    assert ops._library_split(x[:200], w) == 0     # few rows: never split
-    assert ops._library_split(x, w[:30000]) == 0   # fewer columns than one round
+    assert ops.library_split(m, n) == 32768
+    chunked = ops.linear(x, w)
+    assert chunked.is_contiguous() and chunked.shape == (m, n)
+    close(chunked, want, 3e-2, 3e-2)
+    assert torch.equal(chunked, HipOps().linear(x, w))   # nothing measured, nothing remembered
+    ops.library_split_min_rows = 0                 # switched off: one call
+    assert ops.library_split(m, n) == 0
+    close(ops.linear(x, w), want, 3e-2, 3e-2)
+    ops = HipOps()
+    assert ops.library_split(200, n) == 0          # few rows: never split
+    assert ops.library_split(m, 30000) == 0        # fewer columns than one round
+    assert ops.library_split(2048, 19456) == 16384 and ops.library_split(2048, 24576) == 0   # 2.4 rounds; 3 whole ones
 
 
 def test_float32_weight_with_bfloat16_activations_stays_float32(ops):

@@ -485,7 +485,8 @@ def test_toy_architecture_from_its_configuration_alone(toy_folder):
     from safetensors.torch import save_file
 
     with tempfile.TemporaryDirectory() as folder:
-        save_file({d.file_name: src.get(d.file_name).contiguous() for d in model.tensor_decls()},
+        # drawn where the engine drew them: a seed's values differ between devices
+        save_file({d.file_name: src.get(d.file_name, DEV).cpu().contiguous() for d in model.tensor_decls()},
                   f"{folder}/model.safetensors")
         Path(folder, "config.json").write_text(json.dumps(TOY))
         for p, out in zip(prompts, outs):
