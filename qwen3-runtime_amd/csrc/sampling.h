@@ -40,3 +40,9 @@ extern "C" int qrt_sample(const SampleArgs* args, hipStream_t stream);
 // hipFree or allocating library routine.
 #define QRT_SAMPLE_SCRATCH_BYTES (64 * 1024)
 extern "C" int qrt_sample_noalloc(const SampleArgs* args, hipStream_t stream);
+
+// Looks the built-in buffer's address up for the current device now (once per device; later calls
+// return at once), so that the first qrt_sample_noalloc on that device, which may sit inside a
+// stream capture, makes no runtime query. Optional: qrt_sample_noalloc does the same at its first
+// call on a device. Returns 0, or -1 with qrt_last_error().
+extern "C" int qrt_sample_noalloc_setup();

@@ -55,6 +55,9 @@ class DecodeGraph:
         self._row_index = None
         self._prepared = False  # the host buffer holds the step after the one launched last
         self._ahead = None      # (requests, lengths, epoch) of a step launched before it was asked for
+        # the ids that step was fed, brought to the host beside it: the step asked for must bring the same
+        self._ahead_ids: torch.Tensor | None = None
+        self._ahead_ids_here = torch.cuda.Event()
 
     def _fill(self, entries: Sequence[StepEntry]):
         runner = self.runner
@@ -174,6 +177,10 @@ class DecodeGraph:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
         self.views_dev["ids"].copy_(tokens)
+        if self._ahead_ids is None:
+            self._ahead_ids = torch.empty(self.batch, dtype=torch.int32, pin_memory=True)
+        self._ahead_ids.copy_(tokens, non_blocking=True)  # a few bytes, on their way before the step's kernels
+        self._ahead_ids_here.record()
         self.runner.last_row_slots = self.views_dev["row_slots"]
         self.graph.replay()
         self._ahead = (list(self._last_rids), list(self._last_starts), self._last_epoch, self.runner.steps_begun)
@@ -191,9 +198,14 @@ class DecodeGraph:
             # the very next step of the runner (no other has used the graphs' shared memory since),
             # for the same requests at the same lengths, owning the same pages
             if ahead == (rids, [runner.cache.length(r) for r in rids], runner.cache.epoch, runner.steps_begun - 1):
-                runner.last_row_slots = self.views_dev["row_slots"]
-                runner.steps_ahead[1] += 1
-                return self.logits  # launched already, with the ids these entries bring
+                # ... and fed the ids these entries bring (they came to the host beside the launch;
+                # whoever waited for the sampled ids has waited for these too). Other ids: the
+                # launched step is one nobody asked for, and this one runs as any other.
+                self._ahead_ids_here.synchronize()
+                if self._ahead_ids.tolist() == [e.tokens[0] for e in entries]:
+                    runner.last_row_slots = self.views_dev["row_slots"]
+                    runner.steps_ahead[1] += 1
+                    return self.logits
         packed = self._fill(entries)
         if self.graph is None:
             if self.ctx is None:

@@ -69,6 +69,12 @@ class Scheduler:
 
     # ---- one step's decision ---------------------------------------------------------
     def schedule(self) -> list[Request]:
+        # Pages that a replayed decode step took ahead for its requests' next tokens go back to the
+        # pool before anybody is offered anything, whenever somebody besides a decoding resident
+        # wants pages (residents are walked first and take theirs again): what a candidate is
+        # offered then never depends on what the step function did ahead of the books.
+        if self.queue or any(self.behind(r) > 1 for r in self.residents):
+            self.cache.trim()
         while True:
             step = self._walk()
             if step:

@@ -643,3 +643,32 @@ def test_sampler_with_an_excluded_id():
     assert lp[0] == pytest.approx(float(torch.log_softmax(biased[0], -1)[8]), abs=1e-5)
     assert tok[1] != 1 and math.isfinite(lp[1])
     assert lp[1] == pytest.approx(float(torch.log_softmax(biased[1], -1)[tok[1]]), abs=1e-4)
+
+
+def test_a_step_launched_ahead_with_other_ids_is_not_the_step_asked_for(model_folders):
+    """``ModelRunner.step_ahead`` launches the next decode step with ids on the device; the next
+    ``step`` finds its logits computed only if it brings those ids. With other ids it runs as any
+    step does, and gives the logits of the ids it was given."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.batch import StepEntry
+    from qwen3_runtime_amd.engine.factory import load
+
+    cfg, w = P.read_model(model_folders["tiny_b"])
+    prompt = prompts_for(cfg, [20], seed=3)[0]
+    follow = [7, 11, 13, 17, 19, 23]
+    loaded = load(model_folders["tiny_b"], EngineConfig(page_size=8, num_pages=16, max_num_seqs=2, dtype="float32",
+                                                        device=DEV, hip_graph=True))
+    runner = loaded.runner
+    loaded.cache.admit("r")
+    runner.step([StepEntry("r", prompt, [len(prompt) - 1])])
+    got = []
+    for i, tok in enumerate(follow):
+        got.append(runner.step([StepEntry("r", [tok], [0])])[0].float().cpu())
+        if i + 1 < len(follow) and i >= 2:  # graphs replay from the third decode step on
+            # odd steps: the ids the next step will bring; even steps: other ids
+            fed = follow[i + 1] if i % 2 else (follow[i + 1] + 1) % cfg["vocab_size"]
+            assert runner.step_ahead(torch.tensor([fed], dtype=torch.int32, device=DEV))
+    launched, taken = runner.steps_ahead
+    assert launched == 3 and taken == 1, (launched, taken)
+    want = P.forward(cfg, w, prompt + follow)[len(prompt):]
+    torch.testing.assert_close(torch.stack(got), want.float(), atol=5e-5, rtol=5e-5)

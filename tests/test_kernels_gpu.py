@@ -600,6 +600,67 @@ def test_decode_attention_ignores_what_a_page_held_before(ops, nq, nkv, d, ps, w
         close(ops.decode_attention(qkv, cache, ctx, nq, nkv, d, scale, window, qw, kw, 1e-6, inv), want, 2e-2, 2e-2)
 
 
+@pytest.mark.parametrize("window,ps", [(40, 16), (33, 8), (None, 16)])
+def test_decode_attention_at_the_windows_edge_and_the_tokens_own_key(ops, window, ps):
+    """The one-kernel decode step with keys made to stand out: the key just outside the window
+    (which would take all the weight if it were seen), the first key inside it, the last cached
+    key and the token's own key (from the product, not from the cache), each with a value of its
+    own, among faint others. A mask that is off by one at either end moves the output by a large
+    part of a value, not by one part in ``window``. Contexts that end around blocks of 32 keys
+    and around pages, the keys in one piece and cut over blocks."""
+    nq, nkv, d = 8, 2, 64
+    first = (window or 40) + 1
+    kvs = [first, first + 1, 64, 65, 72, 73, 96, 97, 128, 129, 300, 1000]
+    seqs = [(1, kv) for kv in kvs]
+    _, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, window=window, seed=7)
+    t = len(seqs)
+    g = torch.Generator().manual_seed(3)
+    u = torch.zeros(d)
+    u[5] = 1.0
+    cache.k.copy_((0.1 * torch.randn(cache.k.shape, generator=g)).to(torch.bfloat16))
+    cache.v.copy_(torch.randn(cache.v.shape, generator=g).to(torch.bfloat16))
+    table = cache.group.block_table.cpu()
+    place = lambda s, pos: (int(table[s, pos // ps]), pos % ps)
+    values = (3 * torch.randn(4, d, generator=g)).to(torch.bfloat16)
+    for s, kv in enumerate(kvs):
+        me = kv - 1
+        marks = [(me - 1, 6.0, values[2])]                                  # the last cached key
+        if window is not None:
+            marks += [(me - window, 12.0, values[0]), (me - window + 1, 6.0, values[1])]   # outside, just inside
+        for pos, strength, value in marks:
+            page, off = place(s, pos)
+            cache.k[page, :, off, :] = (strength * u).to(torch.bfloat16)
+            cache.v[page, :, :, off] = value
+    qkv = torch.zeros(t, (nq + 2 * nkv) * d)
+    qkv[:, : nq * d] = (8.0 * u).repeat(nq)                                 # scores are then the strengths
+    qkv[:, nq * d: (nq + nkv) * d] = (6.0 * u).repeat(nkv)                  # the token's own key
+    qkv[:, (nq + nkv) * d:] = values[3].float().repeat(nkv)
+    qkv = qkv.to(torch.bfloat16).to(DEV)
+    slots = torch.tensor([place(s, kv - 1)[0] * ps + place(s, kv - 1)[1] for s, kv in enumerate(kvs)],
+                         dtype=torch.int32, device=DEV)
+    cache.group.slots = slots
+    scale = 1.0 / math.sqrt(d)
+    before_k, before_v = cache.k.clone(), cache.v.clone()
+
+    def plain(win):
+        k, v = before_k.clone(), before_v.clone()
+        q = R.qk_norm_rope_store(qkv, nq, nkv, d, None, None, 0.0, None, ctx.positions, k, v, slots, ps)
+        return R.paged_attention(q, k, v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table, ps, nq, nkv, d,
+                                 scale, win).float()
+
+    want = plain(window)
+    if window is not None:  # what a mask off by one at the window's edge would give is far away
+        assert float((plain(window + 1) - want).abs().max()) > 1.0 and float((plain(window - 1) - want).abs().max()) > 0.5
+    assert ops.fuses_decode_attention(ctx, qkv, nq, nkv, d, cache)
+    for splits in (None, 1, 2, 5):
+        cache.k.copy_(before_k)
+        cache.v.copy_(before_v)
+        ctx.scratch.pop("attn_splits", None)
+        if splits:
+            ctx.scratch["attn_splits"] = splits
+        close(ops.decode_attention(qkv, cache, ctx, nq, nkv, d, scale, window, None, None, 0.0, None), want, 3e-2, 2e-2)
+
+
 def test_paged_attention_splits_agree(ops):
     """Long single sequences split over many blocks; empty splits must not leak."""
     seqs, nq, nkv, d, ps = [(1, 2100), (1, 40), (3, 900)], 8, 2, 64, 16

@@ -182,6 +182,7 @@ def test_nothing_running_and_no_page_is_an_error():
     s.add(Request(list(range(5)), max_tokens=2))
     s.cache.admit("squatter")
     s.cache.reserve("squatter", 8)
+    s.cache.commit("squatter", 8)   # stored tokens: pages held only ahead of the books would go back
     with pytest.raises(RuntimeError, match="cannot get a cache page"):
         s.schedule()
 
@@ -269,3 +270,23 @@ def test_a_windowed_model_serves_requests_longer_than_its_pool():
     # a model that keeps every key refuses the same request in the same pool
     with pytest.raises(RuntimeError, match="needs 50 cache pages"):
         scheduler(num_pages=5, page_size=4).add(Request(list(range(150)), max_tokens=50))
+
+
+def test_pages_held_ahead_do_not_change_what_a_prompt_is_offered():
+    """A replayed decode step reserves the page of its request's next token while the device runs.
+    In a pool at its peak such a page must not shorten a queued prompt's portion: the plan is the
+    one made with the books as the last step left them."""
+    def plan(reserve_ahead):
+        s = scheduler(num_pages=4, page_size=4, budget=32)
+        a = Request(list(range(4)), max_tokens=8)
+        s.add(a)
+        run(s, s.schedule(), [9])                       # a holds one page, full; its next token needs a second
+        if reserve_ahead:
+            s.cache.reserve(a.request_id, 1)            # what the step function does ahead of the books
+        b = Request(list(range(100, 108)), max_tokens=2)
+        s.add(b)
+        batch = s.schedule()
+        s.cache.check()
+        return [(r is a, r.grant) for r in batch], s.cache.num_free_pages
+
+    assert plan(True) == plan(False) == ([(True, 1), (False, 8)], 0)

@@ -70,6 +70,10 @@ def _same(got, want):
 def test_no_alloc_sampling_equals_the_existing_entry_point_twice_in_a_row():
     lib, _, _ = _library()
     lib.qrt_last_error.restype = ctypes.c_char_p
+    torch.zeros(1, device=DEV)  # the device is current in this thread
+    # set-up ahead of the first call, as a caller under stream capture would; again is harmless
+    assert lib.qrt_sample_noalloc_setup() == 0, lib.qrt_last_error().decode()
+    assert lib.qrt_sample_noalloc_setup() == 0
     # first call: 12 rows in 21 parts each; second, right after it: 5 rows of a shorter vocabulary
     # in 9 parts, which finds the first call's results still in the built-in buffer
     for rows, vocab, parts, seed in ((12, 50_000, 21, 1), (5, 20_480, 9, 2)):
