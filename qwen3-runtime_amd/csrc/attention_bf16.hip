@@ -62,7 +62,8 @@ struct AttnTileArgs {
   int table_width, num_tiles, nq, nkv, page_size, window, num_splits, waves;
   float scale_log2;
   int row_tiles;  // tiles of 16 rows per wave (general kernel): 1, 2 or 4
-  int use_lds;    // long portions: share keys and values of a block of waves through LDS
+  int use_lds;    // long portions: share keys and values of a block of waves through LDS (1), and
+                  // cut the blocks of keys between two groups of four waves in one block (2)
   // a launch that covers only some of the step's sequences (the others go to another kernel):
   // the tokens whose rows the merge of key splits may write; null: all rows
   const int* merge_tokens;
@@ -483,10 +484,23 @@ __device__ __forceinline__ void tile_probabilities(const f32x4_t sc[2], float sc
 constexpr int VROW = 48;                        // elements per value row (one head element, 32 keys) in LDS
 constexpr int STAGE_ELEMS = 32 * KROW + D * VROW;
 
-template <int RT, bool P2>
-__global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTileArgs a) {
-  extern __shared__ bf16_t lds_kv[];  // [2][STAGE_ELEMS]
-  const int lane = threadIdx.x & 63, wave = uniform_wave_number();
+//
+// G = 2: eight waves, two groups of four that both own the block's rows and take the blocks of
+// keys in turn (group 0 the even ones of the block's range, group 1 the odd ones), each with LDS
+// stages, running maxima, sums and accumulators of its own; at the end group 1 hands its sums
+// over through LDS and group 0 joins them. A causal prompt without history is a triangle: the row
+// tile at its end walks 64 blocks of keys at 2,048 tokens, the one at its start one, and a wave's
+// round is a chain (products, maxima, exponentials, products) that another wave on the SIMD
+// hides only in part: a block alone on its compute unit walked a round in 0.78 of the time it
+// takes beside a second block. So the longest tile alone set the kernel's time (64 rounds; 72 us
+// where an even spread of the rounds over the compute units would take 48). Cut this way the
+// longest chain is half as long, a compute unit holds one block of eight waves at a time, and
+// the blocks, longest first, are dealt out as compute units fall free.
+template <int RT, bool P2, int G>
+__global__ __launch_bounds__(256 * G, G == 1 ? 2 : 1) void attention_bf16_prefill_kernel(AttnTileArgs a) {
+  extern __shared__ bf16_t lds_kv[];  // [G][2][STAGE_ELEMS]
+  const int lane = threadIdx.x & 63, wave_of_block = uniform_wave_number();
+  const int grp = G == 1 ? 0 : wave_of_block >> 2, wave = G == 1 ? wave_of_block : wave_of_block & 3;
   const int r16 = lane & 15, quad = lane >> 4;
   const int tile = blockIdx.x / a.nkv, kvh = blockIdx.x - tile * a.nkv, split = blockIdx.z;
   const int seq = a.tile_seq[tile];
@@ -585,7 +599,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
     }
   };
   auto stash = [&](int b, int stage, const Pieces& in) {  // registers -> LDS: block b into its stage
-    bf16_t* kb = lds_kv + stage * STAGE_ELEMS;
+    bf16_t* kb = lds_kv + (2 * grp + stage) * STAGE_ELEMS;
     bf16_t* vb = kb + 32 * KROW;
     // values of keys no row of the block sees were read from a clamped place, or lie after the
     // sequence's last key in its last page: they may be anything, and 0 * NaN is NaN, so they
@@ -617,12 +631,14 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   // long as a load that hits in L2: with one round of lead the store to LDS sometimes waited for
   // it; measured 2 to 7 % off the kernel's time). Set A carries the blocks of even rounds, set B
   // those of odd rounds; a set is free again once its block has been stored.
-  const int b_first = min(b0, all_b1 - 1);
+  // A group's blocks are b0 + grp, b0 + grp + G, ...; every group runs the rounds of the one
+  // with the most blocks (the barriers are the whole block's), the last of them idle if need be.
+  const int b_first = min(b0 + grp, all_b1 - 1);
   const int b_last = max(b1 - 1, b_first);  // loads past the end repeat the last block and are not used
   auto multiply = [&](int b, int stage) {
     if (b >= wb0 && b < wb1) {  // uniform over the wave
       const int base = b << 5;
-      const bf16_t* kb = lds_kv + stage * STAGE_ELEMS;
+      const bf16_t* kb = lds_kv + (2 * grp + stage) * STAGE_ELEMS;
       const bf16_t* vb = kb + 32 * KROW;
       bf16x8_t kk[2][KFULL > 0 ? KFULL : 1], kt[2];
 #pragma unroll
@@ -694,28 +710,61 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
   };
   int page = lookup(b_first);
   fetch(b_first, page, set_a);
-  page = lookup(min(b0 + 1, b_last));
+  page = lookup(min(b0 + grp + G, b_last));
   stash(b_first, 0, set_a);
-  fetch(min(b0 + 1, b_last), page, set_b);
-  page = lookup(min(b0 + 2, b_last));
+  fetch(min(b0 + grp + G, b_last), page, set_b);
+  page = lookup(min(b0 + grp + 2 * G, b_last));
   __syncthreads();
-  for (int b = b0; b < b1; b += 2) {
-    // even round: set A is free, set B holds block b + 1
-    fetch(min(b + 2, b_last), page, set_a);
-    page = lookup(min(b + 3, b_last));
+  for (int round = b0; round < b1; round += 2 * G) {
+    const int b = round + grp;  // this group's block of the even round; b + G the odd round's
+    // even round: set A is free, set B holds block b + G
+    fetch(min(b + 2 * G, b_last), page, set_a);
+    page = lookup(min(b + 3 * G, b_last));
     multiply(b, 0);
-    stash(min(b + 1, b_last), 1, set_b);
+    stash(min(b + G, b_last), 1, set_b);
     __syncthreads();
-    // odd round: set B is free, set A holds block b + 2. With an odd number of blocks the last
-    // odd round has nothing to multiply (b + 1 == b1 lies outside every wave's range) and only
+    // odd round: set B is free, set A holds block b + 2 G. With an odd number of blocks the last
+    // odd round has nothing to multiply (b + G >= b1 lies outside every wave's range) and only
     // fetches and stores the last block once more. Leaving the loop here instead gave the
     // compiler a path back to the loop's head with set A's loads in flight, and made it wait
     // for every load at the head of every round.
-    fetch(min(b + 3, b_last), page, set_b);
-    page = lookup(min(b + 4, b_last));
-    multiply(b + 1, 1);
-    stash(min(b + 2, b_last), 0, set_a);
+    fetch(min(b + 3 * G, b_last), page, set_b);
+    page = lookup(min(b + 4 * G, b_last));
+    multiply(b + G, 1);
+    stash(min(b + 2 * G, b_last), 0, set_a);
     __syncthreads();
+  }
+
+  if constexpr (G == 2) {
+    // Group 1 hands its reference maxima, sums and accumulators to group 0, lane to lane (the two
+    // hold the same rows in the same lanes), through the LDS the stages no longer need (the loop's
+    // last barrier lies behind every read of them). Both references are lazy ones, below the
+    // rows' maxima by 2^LAZY at most; the join takes the larger and shrinks the other side.
+    f32x4_t* xo = (f32x4_t*)lds_kv;                                 // [4 waves][RT][DB][64 lanes]
+    float* xm = (float*)(xo + 4 * RT * DB * 64);                    // [4 waves][RT][2][64 lanes]
+    if (grp == 1) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+#pragma unroll
+        for (int i = 0; i < DB; ++i) xo[((wave * RT + t) * DB + i) * 64 + lane] = o[t][i];
+        xm[((wave * RT + t) * 2 + 0) * 64 + lane] = m[t];
+        xm[((wave * RT + t) * 2 + 1) * 64 + lane] = l[t];
+      }
+    }
+    __syncthreads();
+    if (grp == 0) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const float m1 = xm[((wave * RT + t) * 2 + 0) * 64 + lane], l1 = xm[((wave * RT + t) * 2 + 1) * 64 + lane];
+        const float m_new = max2(m[t], m1);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float f0 = __builtin_amdgcn_exp2f(m[t] - m_use), f1 = __builtin_amdgcn_exp2f(m1 - m_use);
+        m[t] = m_new;
+        l[t] = l[t] * f0 + l1 * f1;
+#pragma unroll
+        for (int i = 0; i < DB; ++i) o[t][i] = o[t][i] * f0 + xo[((wave * RT + t) * DB + i) * 64 + lane] * f1;
+      }
+    }
   }
 
 #pragma unroll
@@ -723,7 +772,7 @@ __global__ __launch_bounds__(256, 2) void attention_bf16_prefill_kernel(AttnTile
     float lt = l[t];
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
-    if (!row_valid[t] || !wave_has_rows) continue;
+    if (!row_valid[t] || !wave_has_rows || grp != 0) continue;
     const float inv = lt > 0.f ? 1.0f / lt : 0.f;
     if (a.num_splits == 1) {
       bf16_t* op = a.out + row_index[t] * D;
@@ -1154,10 +1203,28 @@ extern "C" int qrt_attention_bf16(const AttnTileArgs* args, int num_rows_total, 
   // the kernel that shares keys and values through LDS, where its two stages fit what a block
   // may have without asking (64 KB: head sizes up to 208); the general kernel otherwise
   constexpr size_t lds_bytes = 2 * (size_t)STAGE_ELEMS * sizeof(bf16_t);
-  if (a.row_tiles == 2 && a.waves == 4 && a.use_lds && lds_bytes <= 64 * 1024) {
+  if (a.row_tiles == 2 && a.waves == 4 && a.use_lds == 2 && lds_bytes <= 64 * 1024) {
+    // two groups of four waves: twice the stages, more LDS than a block gets without asking
+    // ... or what the join of the two groups' sums needs afterwards, in the same memory (more than
+    // the stages at small head sizes): accumulators [4 waves][2 tiles][DB][64 lanes] of 16 bytes,
+    // maxima and sums [4][2][2][64] of 4
+    constexpr size_t join_bytes = (size_t)4 * 2 * DB * 64 * 16 + (size_t)4 * 2 * 2 * 64 * 4;
+    constexpr size_t smem = 2 * lds_bytes > join_bytes ? 2 * lds_bytes : join_bytes;
+    static bool allowed = false;  // once: not again inside every stream capture
+    if (!allowed) {
+      if (hipFuncSetAttribute((const void*)attention_bf16_prefill_kernel<2, true, 2>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess ||
+          hipFuncSetAttribute((const void*)attention_bf16_prefill_kernel<2, false, 2>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+        return qrt_fail("attention (long portions, two groups): cannot get %zu bytes of LDS", smem);
+      allowed = true;
+    }
+    if (p2) attention_bf16_prefill_kernel<2, true, 2><<<grid, dim3(512), smem, stream>>>(a);
+    else attention_bf16_prefill_kernel<2, false, 2><<<grid, dim3(512), smem, stream>>>(a);
+  } else if (a.row_tiles == 2 && a.waves == 4 && a.use_lds && lds_bytes <= 64 * 1024) {
     const size_t smem = lds_bytes;
-    if (p2) attention_bf16_prefill_kernel<2, true><<<grid, block, smem, stream>>>(a);
-    else attention_bf16_prefill_kernel<2, false><<<grid, block, smem, stream>>>(a);
+    if (p2) attention_bf16_prefill_kernel<2, true, 1><<<grid, block, smem, stream>>>(a);
+    else attention_bf16_prefill_kernel<2, false, 1><<<grid, block, smem, stream>>>(a);
   } else if (a.row_tiles == 1 && p2) attention_bf16_kernel<1, true><<<grid, block, 0, stream>>>(a);
   else if (a.row_tiles == 1) attention_bf16_kernel<1, false><<<grid, block, 0, stream>>>(a);
   else if (a.row_tiles == 2 && p2) attention_bf16_kernel<2, true><<<grid, block, 0, stream>>>(a);

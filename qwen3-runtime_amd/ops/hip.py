@@ -181,6 +181,9 @@ class HipOps:
     prefill_row_tiles = 2
     # long portions: keys and values go through LDS, shared by the four waves of a block
     prefill_through_lds = True
+    # ... in blocks of eight waves, two groups that take the blocks of keys in turn: 1 never, 2 always,
+    # None where the longest tile's chain of rounds would otherwise set the kernel's time
+    prefill_key_groups = None
 
     def __init__(self):
         self.lib = core_library()
@@ -608,6 +611,39 @@ class HipOps:
         row0 = [r for _, _, r in items]
         return np.asarray(seqs + row0, dtype=np.int32), len(seqs)
 
+    def choose_key_groups(self, q_lens, kv_lens, group_size: int, nkv: int, window: int, forced_splits=None) -> int:
+        """Long portions through LDS: blocks of four waves, two to a compute unit (1), or blocks of
+        eight waves whose two halves take the blocks of keys in turn (2). A tile of 128 rows walks
+        its keys in rounds of 32, one after the other, and a lone block's round takes 0.78 of what
+        it takes beside a second block: where the tile with the most rounds has about as many as a
+        compute unit gets from all tiles together, that chain sets the kernel's time, and halving
+        it pays although the eight waves, which meet at one barrier, walk a round more slowly than
+        two blocks of four. Measured at head size 128 with 32 query heads on 8 key heads (two
+        groups against one): a 2,048-token prompt 63 against 69 us; prompts of 1,024 tokens with
+        0 and 1,976 tokens before them 83 against 98; portions of 700, 900 and 448 tokens with
+        0, 400 and 4,552 before them 104 against 145; 2,048 tokens with 1,024 before them level;
+        with 2,048 before them 148 against 142. Where the keys are cut over blocks anyway (few
+        tiles), they are not cut again."""
+        if self.prefill_key_groups is not None:
+            return self.prefill_key_groups
+        rounds = longest = tiles = 0
+        for n, kv in zip(q_lens, kv_lens):
+            first = kv - n
+            for r in range(0, n * group_size, 128):
+                hi = first + (min(n * group_size, r + 128) - 1) // group_size
+                lo = max(0, first + r // group_size - window + 1) if window else 0
+                t = (hi >> 5) - (lo >> 5) + 1
+                rounds += t
+                longest = max(longest, t)
+                tiles += 1
+        splits = forced_splits or self.choose_splits(tiles, nkv, max(kv_lens))
+        if splits > 1:
+            return 1
+        return 2 if longest > self.key_groups_ratio * rounds * nkv / 256 else 1
+
+    # see choose_key_groups: the longest tile's rounds over the mean rounds of a compute unit
+    key_groups_ratio = 0.9
+
     @staticmethod
     def choose_splits(num_tiles: int, nkv: int, max_kv: int) -> int:
         """Portions: how many ways to split the keys so that few long sequences still fill the chip."""
@@ -674,18 +710,21 @@ class HipOps:
                 tiles = None if subset is None else torch.tensor(subset, dtype=torch.int32, device=dev)
                 n_tiles = len(q_lens)
             else:
+                lds = waves == 4 and row_tiles >= 2 and self.prefill_through_lds
+                groups = self.choose_key_groups(q_lens, kv_lens, g, nkv, window,
+                                                ctx.scratch.get("attn_splits")) if lds else 0
                 host, n_tiles = self.plan_tiles(q_lens, kv_lens, g, 16 * waves * row_tiles, nkv,
-                                                self.resident_blocks if waves == 4 and row_tiles >= 2 else 0,
-                                                subset)
+                                                self.resident_blocks if waves == 4 and row_tiles >= 2 and groups < 2
+                                                else 0, subset)
                 tiles = torch.from_numpy(host).to(dev)
             tokens = None
             if subset is not None:  # the tokens of these sequences: where a merge of key splits may write
                 cu = np.concatenate([[0], np.cumsum(ctx.q_lens_host)])
                 tokens = torch.from_numpy(np.concatenate([np.arange(cu[s], cu[s + 1]) for s in subset])
                                           .astype(np.int32)).to(dev)
-            plan = (tiles, n_tiles, tokens)
+            plan = (tiles, n_tiles, tokens, 0 if decode else groups)
             ctx.scratch[key] = plan
-        tiles, n_tiles, tokens = plan
+        tiles, n_tiles, tokens, groups = plan
         splits = ctx.scratch.get("attn_splits") or (
             self.choose_decode_splits(n_tiles, nkv, max_kv) if decode else self.choose_splits(n_tiles, nkv, max_kv))
         a = _AttnTileArgs()
@@ -707,7 +746,7 @@ class HipOps:
             a.merge_tokens, a.num_merge_tokens = tokens.data_ptr(), tokens.numel()
         a.num_tiles, a.nq, a.nkv, a.page_size, a.window = n_tiles, nq, nkv, cache.group.page_size, window
         a.num_splits, a.waves, a.row_tiles = splits, waves, row_tiles
-        a.use_lds = 1 if self.prefill_through_lds else 0
+        a.use_lds = groups
         a.scale_log2 = scale * math.log2(math.e)
         if splits > 1:
             part_o = torch.empty((ctx.num_tokens * nq * splits, d), dtype=torch.float32, device=out.device)

@@ -689,6 +689,48 @@ def test_long_portions_split_over_blocks_agree(ops, seqs, nq, nkv, d, ps, window
         close(got, want, 2e-2, 2e-2)
 
 
+@pytest.mark.parametrize("groups", [1, 2])
+@pytest.mark.parametrize("seqs,nq,nkv,d,ps,window,poison", [
+    ([(300, 300)], 4, 1, 128, 16, None, True),                 # a whole prompt: the triangle
+    ([(129, 129), (90, 1200), (70, 75)], 6, 2, 32, 24, None, True),
+    ([(2048, 2048)], 32, 8, 128, 16, None, False),             # the measured prompt's own shape
+    ([(200, 1000), (65, 65)], 8, 2, 64, 8, 150, True),         # a window: blocks of keys that begin late
+    ([(100, 131)], 5, 1, 80, 40, None, True),                  # a 16-wide remainder of the head size
+    ([(70, 70), (33, 140)], 4, 2, 16, 16, None, True),         # the smallest head size: the join needs more LDS than the stages
+    ([(150, 150)], 3, 1, 48, 8, None, False),
+    ([(260, 2000)], 2, 2, 208, 16, None, False),               # the largest head size whose stages fit
+])
+def test_long_portions_with_the_keys_cut_between_two_groups_of_waves(ops, groups, seqs, nq, nkv, d, ps, window, poison):
+    """Portions of more than 64 rows in blocks of four waves, and in blocks of eight whose halves
+    take the blocks of 32 keys in turn and join their sums at the end: odd and even numbers of
+    key blocks, a group left without any, splits over blocks on top, unwritten places full of NaN."""
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, seed=5, window=window, poison=poison)
+    scale = 1.0 / math.sqrt(d)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, scale, window)
+    ops.prefill_key_groups = groups
+    try:
+        for splits in (None, 1, 2, 3, 40):
+            ctx.scratch.clear()
+            if splits:
+                ctx.scratch["attn_splits"] = splits
+            close(ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, window), want, 2e-2, 2e-2)
+    finally:
+        ops.prefill_key_groups = None
+
+
+def test_which_long_portions_cut_their_keys_between_two_groups(ops):
+    """The choice follows from the step's lengths alone: two groups where the longest tile's rounds
+    reach what a compute unit gets on average, and never on top of a cut over blocks."""
+    pick = lambda seqs, nq=32, nkv=8: ops.choose_key_groups([a for a, _ in seqs], [b for _, b in seqs], nq // nkv, nkv, 0)
+    assert pick([(2048, 2048)]) == 2 and pick([(512, 512)]) == 2
+    assert pick([(700, 700), (900, 1300), (448, 5000)]) == 2
+    assert pick([(2048, 4096)]) == 1 and pick([(2048, 8192)]) == 1       # long histories: every tile is long
+    assert pick([(1024, 1024)]) == 1                                      # few tiles: the keys are cut over blocks
+    assert pick([(2048, 2048)], nq=64) == 1                               # twice the tiles for the same keys
+    assert ops.choose_key_groups([2048], [2048], 4, 8, 0, forced_splits=3) == 1
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_paged_attention_random_shapes(ops, seed):
     """Seeded random mixes of decoded tokens, short and long portions, head counts, head sizes,
