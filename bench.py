@@ -106,23 +106,33 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--preset", default="qwen3_4b")
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--prompt-len", type=int, default=2048)
-    ap.add_argument("--context", type=int, default=8192)
+    ap.add_argument("--preset", default=None, help="default: qwen3_4b (mix: qwen3_8b; capacity: qwen3_32b)")
+    ap.add_argument("--batch", type=int, default=None, help="default 8 (capacity: 32)")
+    ap.add_argument("--prompt-len", type=int, default=None, help="default 2048 (capacity: 16384)")
+    ap.add_argument("--context", type=int, default=None, help="default 8192 (capacity: 32768)")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill measurement")
     ap.add_argument("--no-peaks", action="store_true", help="skip the microbenchmark of the device's own peaks")
     ap.add_argument("--trials", type=int, default=TRIALS, help="timed windows of --steps steps each")
-    ap.add_argument("--workload", default="decode", choices=["decode", "mix"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "mix", "capacity"],
                     help="decode: the closed batch (default). mix: --requests requests with prompts of 128 to 4,096 "
-                         "tokens and 256 output tokens each through the scheduler, prompts read in portions of 2,048")
+                         "tokens and 256 output tokens each through the scheduler, prompts read in portions of 2,048 "
+                         "(the 8B shape unless --preset says otherwise). capacity: the closed batch at the 32B shape, "
+                         "32 prompts of 16,384 tokens with room for 512 outputs each in a context of 32,768, decode "
+                         "steps only (no batch 1 / 64, no single-prompt prefill; the prompts' reading is prompt_phase)")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure only the 2,048-token prefill (for profiling); prints a reduced line")
     args = ap.parse_args()
+    by_workload = {"decode": ("qwen3_4b", 8, 2048, 8192), "mix": ("qwen3_8b", 8, 2048, 8192),
+                   "capacity": ("qwen3_32b", 32, 16384, 32768)}[args.workload]
+    for name, value in zip(("preset", "batch", "prompt_len", "context"), by_workload):
+        if getattr(args, name) is None:
+            setattr(args, name, value)
+    if args.workload == "capacity":
+        args.no_points = True
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine is single-GPU)")
         return 2
