@@ -11,6 +11,7 @@ from .base import (  # noqa: F401
     Part,
     PositionEncoding,
     StepContext,
+    StepCost,
 )
 from .model import DecoderModel, build_part  # noqa: F401
-from .plan import CacheSpec, LayerSpec, ModelPlan, PartSpec, RunStep, TensorDecl  # noqa: F401
+from .plan import CacheSpec, LayerSpec, ModelPlan, PagedStream, PartSpec, RunStep, TensorDecl  # noqa: F401

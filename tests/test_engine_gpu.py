@@ -213,3 +213,45 @@ def test_trace_run_program(model_folders, tiny_configs, tmp_path, dtype):
         for e in s["entries"]:
             pos[e["id"]] = pos.get(e["id"], 0) + len(e["tokens"])
     check(got, traces.plain_logits(model_folders["tiny_b"], reqs), dtype)
+
+
+def test_trace_run_program_with_a_preset_and_a_page_count(tmp_path):
+    """``--preset NAME --seed S`` in place of a folder and ``--num-pages`` in place of ``--max-tokens``:
+    the logits are those of an engine built in this process from the same registered
+    configuration and seed, stepped the same way."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import build_model, load
+    from qwen3_runtime_amd.registry import preset_config
+    from qwen3_runtime_amd.weights import RandomSource
+
+    raw = preset_config("tiny_a")
+    reqs = traces.make_requests(raw["vocab_size"], [21, 40], seed=8)
+    steps = traces.portions(reqs)
+    pages = traces.peak_tokens(steps, unit=16) // 16
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "trace_run"), "--preset", "tiny_a", "--seed", "6", "--dtype", "float32",
+         "--out", str(out), "--num-pages", str(pages)],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600,
+    )
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    source = RandomSource(build_model(raw)[1].tensor_decls(), 6, norm_jitter=0.1)
+    loaded = load(None, EngineConfig(page_size=16, num_pages=pages, max_num_seqs=4, dtype="float32", device="cuda:0",
+                                     hip_graph=False), source=source, raw_config=raw)
+    want = traces.replay(loaded, steps)
+    pos: dict = {}
+    for s in steps:
+        arr = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(-1, raw["vocab_size"])
+        row = 0
+        for e in s["entries"]:
+            for w in e["want"]:
+                assert torch.equal(torch.from_numpy(arr[row].copy()), want[(e["id"], pos.get(e["id"], 0) + w)])
+                row += 1
+            pos[e["id"]] = pos.get(e["id"], 0) + len(e["tokens"])
+        assert row == arr.shape[0]
+    # neither or both of a pair of options is a usage error
+    for bad in (["--max-tokens", "64"], ["--preset", "tiny_a", "--model", "x", "--max-tokens", "64"],
+                ["--preset", "tiny_a"]):
+        proc = subprocess.run([sys.executable, str(ROOT / "bin" / "trace_run"), "--out", str(out), *bad],
+                              input="", capture_output=True, text=True, timeout=120)
+        assert proc.returncode == 2, (bad, proc.stderr[-500:])

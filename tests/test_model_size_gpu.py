@@ -226,8 +226,10 @@ def test_model_sized_decode_graph_equals_eager(sized):
     (again, graph_logprobs), replayed = run(True, forced=tokens)
     assert replayed, "no decode step was replayed from a graph"
     assert again == tokens
-    for a, b in zip(graph_logprobs, logprobs):
-        torch.testing.assert_close(torch.tensor(a), torch.tensor(b), atol=0.03, rtol=0)
+    # both are bfloat16 with other partial sums: rounding noise in units of the logits' deviation
+    _, want = sized.plain_logits("qwen3_4b", [70, 20, 5], seed=8)
+    std = float(torch.stack(list(want.values())).double().std())
+    traces.compare_logprobs([x for lp in graph_logprobs for x in lp], [x for lp in logprobs for x in lp], std)
 
 
 @pytest.mark.parametrize("name,dtype,copies", [("qwen3_4b", "bfloat16", True), ("qwen3_4b", "float32", True),
