@@ -123,6 +123,8 @@ def main() -> int:
                          "32 prompts of 16,384 tokens with room for 512 outputs each in a context of 32,768, decode "
                          "steps only (no batch 1 / 64, no single-prompt prefill; the prompts' reading is prompt_phase)")
     ap.add_argument("--requests", type=int, default=64)
+    ap.add_argument("--budget", type=int, default=2048, help="tokens per step (max_num_batched_tokens); the workloads "
+                                                             "name 2,048")
     ap.add_argument("--prefill-only", action="store_true",
                     help="measure only the 2,048-token prefill (for profiling); prints a reduced line")
     args = ap.parse_args()
@@ -156,7 +158,7 @@ def main() -> int:
     mix = args.workload == "mix"
     if mix:
         max_batch = args.requests
-    budget = 2048  # tokens per step
+    budget = args.budget  # tokens per step
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     dev_name = "cuda:0"
 
