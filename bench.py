@@ -277,14 +277,12 @@ def main() -> int:
         t = time.perf_counter()
         reqs = [engine.request(engine.add_request(p, max_tokens=256, sampling=SamplingParams())) for p in prompts]
         n_steps = 0
-        floor_s = 0.0  # what the steps that ran would take at the published peaks
+        ran = []  # per step: its spans and the rows it sampled for, priced after the clock stops
         stamps: dict[int, list[float]] = {r.request_id: [] for r in reqs}  # arrival time of every token
         while not engine.is_finished():
             out = engine.step()
             now = time.perf_counter() - t
-            stats = engine.last_step_stats
-            nbytes, flop = step_bytes_and_flop(stats["spans"], sum(tok is not None for _, tok, _ in out))
-            floor_s += max(nbytes / (HBM_PEAK_GBS * 1e9), flop / MFMA_PEAK[dtype_key])
+            ran.append((engine.last_step_stats["spans"], sum(tok is not None for _, tok, _ in out)))
             for rid, tok, _done in out:
                 if tok is not None:
                     stamps[rid].append(now)
@@ -292,6 +290,10 @@ def main() -> int:
         torch.cuda.synchronize(dev)
         dt = time.perf_counter() - t
         out_tokens = sum(len(r.output_tokens) for r in reqs)
+        floor_s = 0.0  # what the steps that ran would take at the published peaks
+        for spans, rows in ran:
+            nbytes, flop = step_bytes_and_flop(spans, rows)
+            floor_s += max(nbytes / (HBM_PEAK_GBS * 1e9), flop / MFMA_PEAK[dtype_key])
         # the reference's closed-batch figures (qwen3_runtime/serving/slo_harness.py:47-87): time to
         # the first token, time per output token after it, gaps between consecutive tokens
         ttft = sorted(ts[0] for ts in stamps.values())
