@@ -731,11 +731,13 @@ def test_which_long_portions_cut_their_keys_between_two_groups(ops):
     assert ops.choose_key_groups([2048], [2048], 4, 8, 0, forced_splits=3) == 1
 
 
+@pytest.mark.parametrize("groups", [None, 2])
 @pytest.mark.parametrize("seed", range(24))
-def test_paged_attention_random_shapes(ops, seed):
+def test_paged_attention_random_shapes(ops, seed, groups):
     """Seeded random mixes of decoded tokens, short and long portions, head counts, head sizes,
     page sizes, windows and key splits against the plain reference: every kernel variant and the
-    edges between them (16, 64 rows; blocks of 32 keys; pages) get hit by some seed."""
+    edges between them (16, 64 rows; blocks of 32 keys; pages) get hit by some seed. Once with the
+    kernels the lengths choose, once with long portions forced into blocks of eight waves."""
     import random
 
     rng = random.Random(1000 + seed)
@@ -758,7 +760,11 @@ def test_paged_attention_random_shapes(ops, seed):
                              ps, nq, nkv, d, scale, window)
     if splits:
         ctx.scratch["attn_splits"] = splits
-    got = ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, window)
+    ops.prefill_key_groups = groups
+    try:
+        got = ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, window)
+    finally:
+        ops.prefill_key_groups = None
     assert torch.isfinite(got.float()).all(), (seqs, nq, nkv, d, ps, window, splits)
     close(got, want, 2e-2, 2e-2)
 
