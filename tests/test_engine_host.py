@@ -160,3 +160,35 @@ def test_default_page_count_is_capped_by_what_requests_can_use(monkeypatch, mode
     monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (200 * 2**30, 288 * 2**30))
     limit = model.plan.max_positions
     assert factory.pages_for_memory(model, cfg, torch.bfloat16, "cuda:0") == 2 * (-(-limit // 8) + 1)
+
+
+def test_bytes_and_operations_of_a_step_come_from_the_plan():
+    """What a measurement prices a step with, for the 4B configuration, against the architecture's
+    own arithmetic: every matrix once (the tied table as the head, not twice), two norm vectors and
+    the q/k norms per layer, the cache of the live requests; a 2,048-token prompt's operations."""
+    from qwen3_runtime_amd.cache import CacheManager
+    from qwen3_runtime_amd.engine.factory import build_model
+    from qwen3_runtime_amd.registry import preset_config
+
+    raw = preset_config("qwen3_4b")
+    _, model = build_model(raw)
+    h, d, i, v, layers = 2560, 128, 9728, 151936, 36
+    q, kv = 32 * d, 8 * d
+    per_layer = h * (q + 2 * kv) + q * h + 3 * h * i
+    weights = 2 * (v * h + layers * (per_layer + 2 * h + 2 * d) + h)
+    decode = model.step_cost([(1, 2090)] * 8, rows=8, elem_bytes=2)
+    assert decode.total_weight_bytes == weights and round(weights / 1e9, 3) == 8.045
+    cache = CacheManager(model.plan.caches, page_size=16, num_pages=2, max_requests=8, device="cpu",
+                         dtype=torch.bfloat16, allocate=False)
+    assert cache.bytes_read([2090] * 8) == 8 * 2090 * 2 * layers * kv * 2          # 147,456 bytes a token
+    assert round((weights + cache.bytes_read([2090] * 8)) / 1e9, 2) == 10.51
+    prompt = model.step_cost([(2048, 2048)], rows=1, elem_bytes=2)
+    attention = 4 * 32 * d * (2048 * 2049 // 2) * layers
+    assert prompt.flop == 2 * 2048 * layers * per_layer + attention + 2 * v * h
+    assert abs(prompt.flop / 1.612e13 - 1) < 1e-3
+    # an untied head: the embedding table is looked up (one row per token), the head is read whole
+    raw8 = preset_config("qwen3_8b")
+    _, model8 = build_model(raw8)
+    cost = model8.step_cost([(1, 100)], rows=1, elem_bytes=2)
+    assert cost.weight_bytes["model.embed_tokens.weight"] == 4096 * 2
+    assert cost.weight_bytes["lm_head.weight"] == 151936 * 4096 * 2
