@@ -29,9 +29,6 @@ class EngineConfig:
     memory_fraction: float = 0.85
     # replay pure-decode steps from captured HIP graphs
     hip_graph: bool = True
-    # keep a second, tile-major copy of every weight matrix for the few-row products of
-    # decoding (faster streaming; costs the matrices' size again)
-    decode_weight_copy: bool = True
 
     def __post_init__(self) -> None:
         if self.page_size < 1:

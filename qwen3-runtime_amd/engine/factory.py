@@ -57,26 +57,6 @@ def pages_for_memory(model: DecoderModel, engine: EngineConfig, dtype: torch.dty
     return max(32, min(useful, int(free * engine.memory_fraction) // per_page))
 
 
-def copies_fit(model: DecoderModel, engine: EngineConfig, dtype: torch.dtype, device) -> bool:
-    """The tile-major weight copies for decoding cost the matrices' size again. They are made only
-    if weights, copies and the cache asked for (or, with the cache sized from what is left, at
-    least as much cache as weights) stay within ``memory_fraction`` of what is free now."""
-    import math
-    import sys
-
-    width = torch.finfo(dtype).bits // 8
-    weights = sum(math.prod(d.shape) for d in model.tensor_decls()) * width
-    per_page = CacheManager.bytes_per_page(model.plan.caches, engine.page_size, width)
-    cache = engine.num_pages * per_page if engine.num_pages else weights
-    free, _total = torch.cuda.mem_get_info(device)
-    if 2 * weights + cache <= free * engine.memory_fraction:
-        return True
-    print(f"[qwen3_runtime_amd] {2 * weights / 1e9:.0f} GB of weights with their decode copies and "
-          f"{cache / 1e9:.0f} GB of cache do not fit in {free * engine.memory_fraction / 1e9:.0f} GB: "
-          f"no decode copies", file=sys.stderr, flush=True)
-    return False
-
-
 def load(model_dir: str | Path | None, engine: EngineConfig, *, source=None, raw_config: dict | None = None,
          ops=None) -> LoadedModel:
     """Build, load and wire up. ``source``/``raw_config`` replace the folder (random weights on
@@ -94,11 +74,7 @@ def load(model_dir: str | Path | None, engine: EngineConfig, *, source=None, raw
         if device.type != "cuda":
             raise RuntimeError("the engine runs on a GPU only; there is no CPU path")
         ops = HipOps()
-    prepare = getattr(ops, "prepare_weight", None) if engine.decode_weight_copy else None
-    if prepare is not None and device.type == "cuda" and not copies_fit(model, engine, dtype, device):
-        prepare = None
-    loader = load_model(model, source, device, dtype, where=f" in {model_dir}" if model_dir else "",
-                        prepare=prepare)
+    loader = load_model(model, source, device, dtype, where=f" in {model_dir}" if model_dir else "")
     num_pages = engine.num_pages or pages_for_memory(model, engine, dtype, device)
     cache = CacheManager(
         model.plan.caches, page_size=engine.page_size, num_pages=num_pages,

@@ -18,7 +18,6 @@ from __future__ import annotations
 
 import ctypes
 import math
-import weakref
 from ctypes import POINTER, Structure, byref, c_float, c_int, c_long, c_void_p
 
 import numpy as np
@@ -166,14 +165,13 @@ class HipOps:
     # gated product, and the product cut along K whose planes the residual's norm adds
     own_max_rows_shared = 128
     # Rows from which a product takes the kernel that shares the activations through LDS
-    # instead of the few-row kernel (both stream tile-major weights). Measured at the 4B
-    # shapes: cut along K the sharing kernel alone is 5 to 22 % faster from 4 rows on, gated
-    # from 12 rows on; a decode step is as fast either way at batch 8 and 5 % faster with it
-    # at batch 16. (Timed on one weight matrix over and over, the sharing kernel looks 15 to
-    # 40 % faster than the few-row kernel down to one row, because a matrix of up to some
-    # 100 MB then stays in the memory-side cache; with the matrices of 36 layers in turn, as in
-    # a step, it is 5 % slower at 8 rows, and a decode step with it from one row on lost 3 % at
-    # batch 8 and 9 % at batch 1.)
+    # instead of the few-row kernel (both stream the weights as stored, through LDS by direct
+    # loads). Measured at the 4B shapes on the matrices of 36 layers in turn: cut along K the
+    # sharing kernel is faster from 9 rows on, gated from 12 rows on. (Timed on one weight
+    # matrix over and over, the sharing kernel looks 15 to 40 % faster than the few-row kernel
+    # down to one row, because a matrix of up to some 100 MB then stays in the memory-side
+    # cache; in a step it is 5 % slower at 8 rows, and a decode step with it from one row on
+    # lost 3 % at batch 8 and 9 % at batch 1.)
     shared_from_rows = {"whole": 17, "gated": 12, "planes": 9}
     # steps of single tokens: norm, rotation, cache write and attention in one kernel
     fuse_decode = True
@@ -187,30 +185,6 @@ class HipOps:
 
     def __init__(self):
         self.lib = core_library()
-        # tile-major copies of weight matrices for the few-row products: address -> (weight, copy)
-        self._tiled: dict[int, tuple] = {}
-
-    # ---- weights prepared for decoding ------------------------------------------
-    def prepare_weight(self, w: torch.Tensor) -> None:
-        """Keep a tile-major copy of ``w`` [N, K] for products with at most ``own_max_rows`` rows.
-
-        Tile (r, s) of 16 rows x 32 columns becomes one contiguous KB in the order the MFMA's
-        lanes read it, so a wave's load is eight whole cache lines instead of sixteen halves:
-        measured 13 to 28 % faster on the 4B model's shapes up to 16 rows; the kernel for 17 to
-        64 rows reads nothing else. Costs the matrix's size again."""
-        if w.dtype != torch.bfloat16 or w.dim() != 2 or not w.is_cuda:
-            return
-        n, k = w.shape
-        if n % 16 or k % 32 or w.data_ptr() in self._tiled:
-            return
-        tiled = w.view(n // 16, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
-        self._tiled[w.data_ptr()] = (weakref.ref(w), tiled)
-
-    def _tiled_copy(self, w: torch.Tensor):
-        entry = self._tiled.get(w.data_ptr())
-        if entry is not None and entry[0]() is w:
-            return entry[1]
-        return None
 
     def _check(self, lib, code: int) -> None:
         if code != 0:
@@ -275,8 +249,7 @@ class HipOps:
             return out if (out_f32 or x.dtype == torch.float32) else out.to(x.dtype)
         if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
             raise OpsError(f"linear: no product of {x.dtype} activations with {w.dtype} weights")
-        tiled = self._tiled_copy(w)
-        kernel = self._own_kernel(m, k, tiled, "whole")
+        kernel = self._own_kernel(m, n, k, "whole")
         if kernel is None:
             # many rows: the vendor library; both accumulate in float32
             if out_f32:
@@ -284,7 +257,7 @@ class HipOps:
             return self._library_product(x, w)
         out = torch.empty((m, n), dtype=torch.float32 if out_f32 else torch.bfloat16, device=x.device)
         self._check(self.lib, self.lib.qrt_gemm_bf16(
-            _ptr(x), _ptr(tiled if kernel else w), _ptr(out), F32 if out_f32 else BF16,
+            _ptr(x), _ptr(w), _ptr(out), F32 if out_f32 else BF16,
             c_int(m), c_int(n), c_int(k), c_int(0), c_int(kernel), c_int(1), _stream()))
         return out
 
@@ -323,19 +296,20 @@ class HipOps:
         split = (n // per_round) * per_round
         return split if 0 < split < n else 0
 
-    def _own_kernel(self, m: int, k: int, tiled, form: str) -> int | None:
-        """Which of the library's kernels multiplies ``m`` rows by this weight: 0 the few-row
-        kernel on the weight as stored, 1 the same on the tile-major copy, 2 the kernel that
-        shares the activations through LDS (tile-major copy, K a multiple of 64), None the
-        vendor library. ``form``: "whole", "gated", or "planes" (cut along K). Measured at the
-        4B shapes against the vendor library: 28 to 32 % less time over the four products of a
-        layer at 32 and 64 rows; at 128 rows 71 us against 116 for the gated product and the
+    def _own_kernel(self, m: int, n: int, k: int, form: str) -> int | None:
+        """Which of the library's kernels multiplies ``m`` rows by a weight [n, k]: 0 the few-row
+        kernel (up to 16 rows), 1 the kernel that shares the activations through LDS (K a
+        multiple of 64 and at least 128, n a multiple of 16), None the vendor library. Both read
+        the weight as stored. ``form``: "whole", "gated", or "planes" (cut along K). Measured at
+        the 4B shapes against the vendor library: 28 to 32 % less time over the four products of
+        a layer at 32 and 64 rows; at 128 rows 71 us against 116 for the gated product and the
         two cut along K."""
         limit = self.own_max_rows if form == "whole" else self.own_max_rows_shared
-        if tiled is not None and k % 64 == 0 and self.shared_from_rows[form] <= m <= limit:
-            return 2
+        if (k % 64 == 0 and k >= 128 and n % 16 == 0 and n <= 1 << 20
+                and self.shared_from_rows[form] <= m <= limit):
+            return 1
         if m <= min(16, limit):
-            return 0 if tiled is None else 1
+            return 0
         return None
 
     def linear_for_residual(self, x, w):
@@ -346,16 +320,19 @@ class HipOps:
         per row tile, which fills the chip (160 row tiles for 256 compute units at the 4B size)."""
         m, k = x.shape
         n = w.shape[0]
-        tiled = self._tiled_copy(w) if x.dtype == torch.bfloat16 else None
-        kernel = self._own_kernel(m, k, tiled, "planes") if tiled is not None else None
-        parts = self.choose_k_parts(n, k, m, kernel == 2) if kernel else 1
+        kernel, parts = None, 1
+        if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and k % 64 == 0:
+            kernel = self._own_kernel(m, n, k, "planes")
+            if kernel is not None:
+                parts = self.choose_k_parts(n, k, m, kernel == 1)
         if parts == 1:
             return self.linear(x, w)
         _need(x, "x", torch.bfloat16)
+        _need(w, "weight", torch.bfloat16, (n, k))
         out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
         self._check(self.lib, self.lib.qrt_gemm_bf16(
-            _ptr(x), _ptr(tiled), _ptr(out), F32, c_int(m), c_int(n), c_int(k), c_int(0), c_int(kernel),
-            c_int(parts), _stream()))
+            _ptr(x), _ptr(w), _ptr(out), F32, c_int(m), c_int(n), c_int(k), c_int(0),
+            c_int(kernel), c_int(parts), _stream()))
         return out
 
     @staticmethod
@@ -370,12 +347,12 @@ class HipOps:
         if not shared:
             if tiles >= 384 or k < 2048:
                 return 1
-            # parts of about 1,024 columns, and about a thousand blocks or more in all, in a
-            # number of planes the residual's norm knows when compiling (timed on the matrices of
-            # 36 layers in turn at the 4B, 8B and 32B sizes: 6 to 13 % less than 2 or 4 parts for
-            # the narrow 4B products, level at the 8B size, 1 to 6 % less at the 32B size)
-            want = max(k // 1024, -(-1024 // tiles))
-            return 2 if want <= 2 else 4 if want <= 4 else 8
+            # four parts up to 8,192 columns and eight beyond, in a number of planes the residual's
+            # norm knows when compiling (timed on the matrices of 36 layers in turn at the 4B, 8B
+            # and 32B sizes: the attention's output product 6.2, 7.6 and 17.6 us in four parts
+            # against 6.8, 8.9 and 18.3 in eight; the down projection 10.6 and 40.6 us in eight
+            # against 12.0 and 43.6 in four at the 4B and 32B sizes, level at the 8B size)
+            return 4 if k <= 8192 else 8
         blocks = (tiles + 5) // 6
         return max(1, min(8, 256 // blocks, (k // 32) // 12))
 
@@ -391,12 +368,11 @@ class HipOps:
         if x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and k % 32 == 0:
             _need(x, "x")
             _need(w_gate_up, "weight")
-            tiled = self._tiled_copy(w_gate_up) if (two_i // 2) % 16 == 0 else None
-            kernel = self._own_kernel(m, k, tiled, "gated")
+            kernel = self._own_kernel(m, two_i // 2, k, "gated")
             if kernel is not None:
                 out = torch.empty((m, two_i // 2), dtype=torch.bfloat16, device=x.device)
                 self._check(self.lib, self.lib.qrt_gemm_bf16(
-                    _ptr(x), _ptr(tiled if kernel else w_gate_up), _ptr(out), BF16, c_int(m),
+                    _ptr(x), _ptr(w_gate_up), _ptr(out), BF16, c_int(m),
                     c_int(two_i // 2), c_int(k), c_int(1), c_int(kernel), c_int(1), _stream()))
                 return out
         return self.swiglu(self.linear(x, w_gate_up))

@@ -35,7 +35,7 @@ from .plan import CacheSpec, TensorDecl
 class WeightFetcher(Protocol):
     """What ``load`` may ask for; implemented by ``weights.loader.WeightLoader``."""
 
-    def matrix(self, file_name: str, linear: bool = True) -> torch.Tensor: ...
+    def matrix(self, file_name: str) -> torch.Tensor: ...
 
     def fused(self, file_names: Sequence[str], dim: int = 0) -> torch.Tensor: ...
 

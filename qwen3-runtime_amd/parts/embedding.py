@@ -27,7 +27,7 @@ class TokenEmbedding(Part):
         return [TensorDecl(self._name("weight"), (self.vocab_size, self.hidden_size), init="embedding")]
 
     def load(self, fetch):
-        self.weight = fetch.matrix(self._name("weight"), linear=False)
+        self.weight = fetch.matrix(self._name("weight"))
 
     def forward(self, ctx, ids):
         return ctx.ops.embed(ids, self.weight)

@@ -75,13 +75,9 @@ def check_source(source, decls: Sequence[TensorDecl], ignorable: Sequence[str] =
 class WeightLoader:
     """Hands device tensors to parts; equal requests share one tensor (tied head)."""
 
-    def __init__(self, source, device: torch.device | str, dtype: torch.dtype, prepare=None):
-        """``prepare(tensor)`` is called once for every matrix that enters a product (the ops may
-        keep a copy of it in a layout of their own)."""
+    def __init__(self, source, device: torch.device | str, dtype: torch.dtype):
         if dtype not in (torch.bfloat16, torch.float32):
             raise ValueError(f"engine dtype must be bfloat16 or float32, got {dtype}")
-        self.prepare = prepare
-        self._prepared: set[int] = set()
         self.source = source
         self.device = torch.device(device)
         self.dtype = dtype
@@ -102,20 +98,12 @@ class WeightLoader:
             self.num_bytes += t.numel() * t.element_size()
         return self._cache[key]
 
-    def _for_products(self, t: torch.Tensor) -> torch.Tensor:
-        if self.prepare is not None and id(t) not in self._prepared:
-            self._prepared.add(id(t))
-            self.prepare(t)
-        return t
-
-    def matrix(self, file_name: str, linear: bool = True) -> torch.Tensor:
-        """``linear=False``: the matrix is only looked up by row (an embedding table)."""
+    def matrix(self, file_name: str) -> torch.Tensor:
         def make():
             t = self.source.get(file_name, self.device)
             return t.to(self._placed_dtype(t.dtype))
 
-        t = self._remember(("matrix", file_name), make)
-        return self._for_products(t) if linear else t
+        return self._remember(("matrix", file_name), make)
 
     def fused(self, file_names: Sequence[str], dim: int = 0) -> torch.Tensor:
         def make():
@@ -125,7 +113,7 @@ class WeightLoader:
             )
             return torch.cat([p.to(target) for p in parts], dim=dim)
 
-        return self._for_products(self._remember(("fused", tuple(file_names), dim), make))
+        return self._remember(("fused", tuple(file_names), dim), make)
 
     def vector_f32(self, file_name: str) -> torch.Tensor:
         return self._remember(
@@ -143,9 +131,9 @@ class WeightLoader:
         return tensor.to(self.device).contiguous()
 
 
-def load_model(model, source, device, dtype, where: str = "", prepare=None) -> WeightLoader:
+def load_model(model, source, device, dtype, where: str = "") -> WeightLoader:
     """Check ``source`` against ``model``'s declarations, then load every part."""
     check_source(source, model.tensor_decls(), model.plan.ignorable, where)
-    loader = WeightLoader(source, device, dtype, prepare)
+    loader = WeightLoader(source, device, dtype)
     model.load(loader)
     return loader

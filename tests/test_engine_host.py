@@ -75,18 +75,16 @@ def test_which_kernel_multiplies_how_many_rows():
     from qwen3_runtime_amd.ops.hip import HipOps
 
     ops = HipOps.__new__(HipOps)          # the choices need no library and no GPU
-    copy = object()                       # stands for a tile-major copy
-    assert [ops._own_kernel(m, 2560, copy, "whole") for m in (1, 16, 17, 64, 65)] == [1, 1, 2, 2, None]
-    assert [ops._own_kernel(m, 2560, copy, "gated") for m in (1, 11, 12, 64, 128, 129)] == [1, 1, 2, 2, 2, None]
-    assert [ops._own_kernel(m, 4096, copy, "planes") for m in (1, 8, 9, 128, 129)] == [1, 1, 2, 2, None]
-    assert [ops._own_kernel(m, 2560, None, "whole") for m in (1, 16, 17)] == [0, 0, None]   # no copy
-    assert [ops._own_kernel(m, 96, copy, "planes") for m in (8, 16, 17)] == [1, 1, None]    # K no multiple of 64
-    # the few-row kernel cuts K when there are few row tiles; the sharing kernel until the chip is full
-    # (parts of about 1,024 columns and about a thousand blocks in all, in 2, 4 or 8 planes: the 4B,
-    # 8B and 32B output and down projections)
-    assert HipOps.choose_k_parts(2560, 4096, 8) == 8 and HipOps.choose_k_parts(2560, 9728, 8) == 8
+    assert [ops._own_kernel(m, 6144, 2560, "whole") for m in (1, 16, 17, 64, 65)] == [0, 0, 1, 1, None]
+    assert [ops._own_kernel(m, 9728, 2560, "gated") for m in (1, 11, 12, 64, 128, 129)] == [0, 0, 1, 1, 1, None]
+    assert [ops._own_kernel(m, 2560, 4096, "planes") for m in (1, 8, 9, 128, 129)] == [0, 0, 1, 1, None]
+    assert [ops._own_kernel(m, 1000, 2560, "whole") for m in (1, 16, 17)] == [0, 0, None]   # rows no multiple of 16
+    assert [ops._own_kernel(m, 2560, 96, "planes") for m in (8, 16, 17)] == [0, 0, None]    # K no multiple of 64
+    # the few-row kernel cuts K when there are few row tiles (four parts up to 8,192 columns, eight
+    # beyond: the 4B, 8B and 32B output and down projections); the sharing kernel until the chip is full
+    assert HipOps.choose_k_parts(2560, 4096, 8) == 4 and HipOps.choose_k_parts(2560, 9728, 8) == 8
     assert HipOps.choose_k_parts(4096, 4096, 8) == 4 and HipOps.choose_k_parts(4096, 12288, 1) == 8
-    assert HipOps.choose_k_parts(5120, 8192, 8) == 8 and HipOps.choose_k_parts(5120, 2048, 8) == 4
+    assert HipOps.choose_k_parts(5120, 8192, 8) == 4 and HipOps.choose_k_parts(5120, 25600, 8) == 8
     assert HipOps.choose_k_parts(6144, 2560, 8) == 1 and HipOps.choose_k_parts(2560, 64, 8) == 1
     assert HipOps.choose_k_parts(2560, 4096, 64) == 8 and HipOps.choose_k_parts(2560, 4096, 12, True) == 8
     assert HipOps.choose_k_parts(2560, 384, 64) == 1 and HipOps.choose_k_parts(65536, 4096, 64) == 1

@@ -280,18 +280,6 @@ def test_engine_refuses_work_after_a_failed_step(model_folders):
         eng.add_request(prompt, 2)
 
 
-def test_decode_weight_copies_only_where_memory_allows(model_folders, capsys):
-    from qwen3_runtime_amd.config.engine import EngineConfig
-    from qwen3_runtime_amd.engine.factory import load
-
-    roomy = load(model_folders["tiny_b"], EngineConfig(page_size=8, num_pages=16, dtype="bfloat16", device=DEV))
-    assert roomy.runner.ops._tiled, "no tile-major copies although memory is plentiful"
-    tight = load(model_folders["tiny_b"], EngineConfig(page_size=8, num_pages=16, dtype="bfloat16", device=DEV,
-                                                       memory_fraction=1e-9))
-    assert not tight.runner.ops._tiled
-    assert "no decode copies" in capsys.readouterr().err
-
-
 def test_requests_arriving_mid_decode_and_seeded_sampling(model_folders):
     """Temperature 0.8 with per-request seeds: tokens do not depend on batch mates or admission time."""
     from qwen3_runtime_amd.sampling.params import SamplingParams

@@ -137,19 +137,16 @@ def test_gated_linear(ops, m, i, k, monkeypatch):
         close(got, want, tol, tol)
 
 
-@pytest.mark.parametrize("prepared", [False, True])
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 32, 40, 64, 65])
 @pytest.mark.parametrize("n,k", [(6144, 2560), (2560, 4096), (1008, 9728), (272, 96), (272, 192)])
-def test_gemm_bf16_few_rows_at_model_sizes(m, n, k, prepared):
-    """Up to 16 rows the few-row kernel, on either weight layout; 17 to 64 rows the kernel that
-    shares the activations through LDS if there is a tile-major copy and K is a multiple of 64;
-    otherwise, and beyond, the vendor library. All of them against a float64 product."""
+def test_gemm_bf16_few_rows_at_model_sizes(m, n, k):
+    """Up to 16 rows the few-row kernel; 17 to 64 rows the kernel that shares the activations
+    through LDS if K is a multiple of 64; otherwise, and beyond, the vendor library. All of them
+    against a float64 product."""
     from qwen3_runtime_amd.ops.hip import HipOps
 
     ops = HipOps()
     x, w = rnd(m, k, dtype=torch.bfloat16, seed=1), rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.02)
-    if prepared:
-        ops.prepare_weight(w)
     want = x.double() @ w.double().T
     got = ops.linear(x, w, out_f32=True)
     assert got.dtype == torch.float32
@@ -161,33 +158,23 @@ def test_gemm_bf16_few_rows_at_model_sizes(m, n, k, prepared):
 @pytest.mark.parametrize("n,k,gated", [(6144, 2560, False), (2560, 4096, False), (608, 9728, False), (64, 64, False),
                                        (9728, 2560, True), (48, 96, True), (151936, 256, False), (80, 128, True),
                                        (4112, 640, True), (16, 64, False)])
-def test_tile_major_weight_copy_gives_the_same_products(m, n, k, gated):
-    """A prepared weight (tile-major copy) gives the products of the plain one: both agree with a
-    float64 product (the two may add partial sums in different orders)."""
+def test_products_of_1_to_128_rows_whole_and_gated(m, n, k, gated):
+    """Every number of rows that changes the kernel (few-row up to 16 rows or below the form's
+    threshold, sharing the activations through LDS beyond, in accumulator blocks of 16 rows up to
+    64 or 128) at shapes with one tile, with fewer tiles than a block takes, with more tiles than
+    compute units, with very many; against a float64 product."""
     from qwen3_runtime_amd.ops.hip import HipOps
 
-    plain, prepared = HipOps(), HipOps()
+    ops = HipOps()
     x = rnd(m, k, dtype=torch.bfloat16, seed=1)
     w = rnd(2 * n if gated else n, k, dtype=torch.bfloat16, seed=2, scale=0.03)
-    prepared.prepare_weight(w)
-    assert prepared._tiled_copy(w) is not None and plain._tiled_copy(w) is None
     if gated:
         want = R.swiglu((x.double() @ w.double().T).to(torch.bfloat16).double())
-        close(prepared.gated_linear(x, w), want, 3e-2, 3e-2)
-        close(plain.gated_linear(x, w), want, 3e-2, 3e-2)
+        close(ops.gated_linear(x, w), want, 3e-2, 3e-2)
     else:
         want = x.double() @ w.double().T
-        close(prepared.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
-        close(plain.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
-        close(prepared.linear(x, w), want, 3e-2, 3e-2)
-    # more rows than the own kernels take: the copy is not used, the result is the library's
-    big = rnd(130, k, dtype=torch.bfloat16, seed=3)
-    if not gated:
-        assert torch.equal(prepared.linear(big, w), plain.linear(big, w))
-    # sizes that cannot be tiled are left alone
-    odd = rnd(24, 48, dtype=torch.bfloat16)
-    prepared.prepare_weight(odd)
-    assert prepared._tiled_copy(odd) is None
+        close(ops.linear(x, w, out_f32=True), want, 2e-3, 2e-3)
+        close(ops.linear(x, w), want, 3e-2, 3e-2)
 
 
 @pytest.mark.parametrize("m", [1, 3, 8, 9, 16, 17, 40, 64, 70, 128, 129])
@@ -199,12 +186,12 @@ def test_product_for_the_residual_may_come_in_planes(m, n, k):
     ops = HipOps()
     x = rnd(m, k, dtype=torch.bfloat16, seed=1)
     w = rnd(n, k, dtype=torch.bfloat16, seed=2, scale=0.03)
-    ops.prepare_weight(w)
     want = x.double() @ w.double().T
     got = ops.linear_for_residual(x, w)
-    kernel = ops._own_kernel(m, k, ops._tiled_copy(w), "planes")
-    parts = ops.choose_k_parts(n, k, m, kernel == 2) if kernel else 1
-    assert (kernel == 2) == (9 <= m <= 128 and k % 64 == 0)
+    kernel = ops._own_kernel(m, n, k, "planes")
+    parts = ops.choose_k_parts(n, k, m, kernel == 1) if kernel is not None and k % 64 == 0 else 1
+    assert (kernel == 1) == (9 <= m <= 128 and k % 64 == 0 and k >= 128)
+    assert (kernel == 0) == (m < 9 or (m <= 16 and k < 128))
     if parts > 1:
         assert got.dim() == 3 and got.shape[0] == parts and got.dtype == torch.float32
         close(got.sum(0), want, 2e-3, 2e-3)
@@ -226,12 +213,50 @@ def test_product_for_the_residual_may_come_in_planes(m, n, k):
     close(yc, ya[rows.long()], 0, 0)
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("n,k,gated", [(1000, 320, False), (50, 64, False), (2560, 4096, False), (4112, 640, True),
+                                       (16, 128, False), (40, 192, True), (6144, 2560, False), (33000, 128, False),
+                                       (640, 5120, False), (9, 2048, True)])
+def test_few_rows_on_weights_as_stored(m, n, k, gated):
+    """The few-row kernel that brings row-major weights through LDS by direct loads, called as the
+    library exports it: any number of weight rows (the last tile repeats the last row), K in pairs
+    of k-steps that do not divide evenly among the waves or the parts, whole and in 2, 4 and 8
+    planes (some of them empty), against a float64 product. A piece of a row in another row's
+    place, or a pair read before it has landed, would show in every entry."""
+    from ctypes import c_int
+
+    from qwen3_runtime_amd.ops.hip import BF16, F32, HipOps, _ptr, _stream
+
+    ops = HipOps()
+    x = rnd(m, k, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * n if gated else n, k, dtype=torch.bfloat16, seed=2, scale=0.03)
+    if gated:
+        want = R.swiglu((x.double() @ w.double().T).to(torch.bfloat16).double())
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops._check(ops.lib, ops.lib.qrt_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), BF16, c_int(m), c_int(n), c_int(k),
+                                                  c_int(1), c_int(0), c_int(1), _stream()))
+        close(out, want, 3e-2, 3e-2)
+        return
+    want = x.double() @ w.double().T
+    for parts in (1, 2, 4, 8):
+        out = torch.full((parts, m, n), float("nan"), dtype=torch.float32, device=DEV)
+        ops._check(ops.lib, ops.lib.qrt_gemm_bf16(_ptr(x), _ptr(w), _ptr(out), F32, c_int(m), c_int(n), c_int(k),
+                                                  c_int(0), c_int(0), c_int(parts), _stream()))
+        close(out.sum(0), want, 2e-3, 2e-3)
+    # planes need the kernel that can cut K: more rows, or a K that is no multiple of 64, are refused
+    with pytest.raises(Exception, match="K parts"):
+        big = rnd(17, k, dtype=torch.bfloat16, seed=3)
+        out = torch.empty((2, 17, n), dtype=torch.float32, device=DEV)
+        ops._check(ops.lib, ops.lib.qrt_gemm_bf16(_ptr(big), _ptr(w), _ptr(out), F32, c_int(17), c_int(n), c_int(k),
+                                                  c_int(0), c_int(0), c_int(2), _stream()))
+
+
 @pytest.mark.parametrize("m", [1, 8, 64])
 def test_vocabulary_head_at_its_real_size(m):
     """The head of the 4B and 8B models, 151,936 x 2,560, through the dispatch a decode step uses
-    (tile-major copy; the few-row kernel with two row tiles per block up to 16 rows, the kernel
-    that shares activations with eight tiles per block for 64), float32 out, against a float64
-    product of the same bfloat16 values computed on the device."""
+    (the few-row kernel with two row tiles per block up to 16 rows; the kernel that shares
+    activations, eight tiles per block, for 64),
+    float32 out, against a float64 product of the same bfloat16 values computed on the device."""
     from qwen3_runtime_amd.ops.hip import HipOps
 
     ops = HipOps()
@@ -239,8 +264,7 @@ def test_vocabulary_head_at_its_real_size(m):
     x = rnd(m, k, dtype=torch.bfloat16, seed=5)
     g = torch.Generator(device=DEV).manual_seed(17)
     w = (0.02 * torch.randn(n, k, generator=g, device=DEV, dtype=torch.float32)).to(torch.bfloat16)
-    ops.prepare_weight(w)
-    assert ops._tiled_copy(w) is not None and ops._own_kernel(m, k, ops._tiled_copy(w), "whole") == (1 if m <= 16 else 2)
+    assert ops._own_kernel(m, n, k, "whole") == (0 if m <= 16 else 1)
     got = ops.linear(x, w, out_f32=True)
     want = torch.empty((m, n), dtype=torch.float64, device=DEV)
     for lo in range(0, n, 16384):                       # in pieces: the float64 copy of W is 3 GB otherwise

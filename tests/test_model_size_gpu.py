@@ -1,10 +1,10 @@
 """The engine at the layer sizes of the 4B, 8B and 32B models (two layers, a small vocabulary; one
 model of the 4B width six layers deep) against the plain implementation: the kernels'
-production paths (few-row products on tile-major weights with K cut into planes, the gated
-epilogue, decode attention at head size 128 with four and eight query heads per key head, prompt
-attention through LDS, the vendor products for long portions, and at the 32B sizes the same
-without tile-major copies, as that model runs) as parts of a whole model, in float32 and
-bfloat16, under every way of cutting the requests into steps.
+production paths (few-row products with K cut into planes, the gated epilogue, the products
+that share their activations through LDS, decode attention at head size 128 with four and eight
+query heads per key head, prompt attention through LDS, the vendor products for long portions)
+as parts of a whole model, in float32 and bfloat16, under every way of cutting the requests into
+steps.
 
 Weights of these widths are drawn on the device and the plain implementation's float64 torch
 routines run there too: the host takes minutes for either."""
@@ -64,13 +64,13 @@ def sized(tmp_path_factory):
     return _Sized(tmp_path_factory)
 
 
-def load_sized(folder, steps, dtype, *, page=16, copies=True, graph=False, max_seqs=4, pages=None, budget=2048):
+def load_sized(folder, steps, dtype, *, page=16, graph=False, max_seqs=4, pages=None, budget=2048):
     from qwen3_runtime_amd.config.engine import EngineConfig
     from qwen3_runtime_amd.engine.factory import load
 
     engine_cfg = EngineConfig(page_size=page, num_pages=pages or -(-traces.peak_tokens(steps) // page),
                               max_num_seqs=max_seqs, max_num_batched_tokens=budget, dtype=dtype, device=DEVICE,
-                              hip_graph=graph, decode_weight_copy=copies)
+                              hip_graph=graph)
     return load(folder, engine_cfg)
 
 
@@ -92,7 +92,6 @@ def test_model_sized_layers_match_plain(sized, name, cut, dtype):
     reqs, want = sized.plain_logits(name, [150, 41, 9], seed=6)
     steps = getattr(traces, cut)(reqs)
     loaded = load_sized(folder, steps, dtype)
-    assert loaded.runner.ops._tiled or dtype == "float32", "the weights have tile-major copies: the own kernels run"
     got = traces.replay(loaded, steps)
     if dtype == "float32":
         traces.compare(got, want, **TOL_F32)
@@ -103,16 +102,13 @@ def test_model_sized_layers_match_plain(sized, name, cut, dtype):
 @pytest.mark.parametrize("dtype,cut", [("float32", "portions"), ("float32", "tail_one_by_one"), ("bfloat16", "whole"),
                                        ("bfloat16", "tail_one_by_one"), ("bfloat16", "portions"),
                                        ("bfloat16", "mixed")])
-def test_32b_layer_sizes_without_decode_copies(sized, dtype, cut):
+def test_32b_layer_sizes(sized, dtype, cut):
     """Width 5,120, 64 query heads on 8 key heads (eight rows of one sequence per decode tile), a
-    feed-forward of 25,600 (the down product's K of 25,600 cut into planes, 1,600 gate/up tiles),
-    and no tile-major copies, as the whole 32B model runs where the copies do not fit: the few-row
-    kernel then reads the weights as stored."""
+    feed-forward of 25,600 (the down product's K of 25,600 cut into planes, 1,600 gate/up tiles)."""
     cfg, folder = sized["qwen3_32b"]
     reqs, want = sized.plain_logits("qwen3_32b", [150, 41, 9], seed=16)
     steps = getattr(traces, cut)(reqs)
-    loaded = load_sized(folder, steps, dtype, copies=False)
-    assert not loaded.runner.ops._tiled
+    loaded = load_sized(folder, steps, dtype)
     got = traces.replay(loaded, steps)
     if dtype == "float32":
         traces.compare(got, want, **TOL_F32)
@@ -120,14 +116,12 @@ def test_32b_layer_sizes_without_decode_copies(sized, dtype, cut):
         check_rounding_noise(got, want)
 
 
-@pytest.mark.parametrize("name,live,copies", [("qwen3_4b", 20, True), ("qwen3_4b", 40, True), ("qwen3_4b", 64, True),
-                                              ("qwen3_8b", 33, True), ("qwen3_32b", 8, False),
-                                              ("qwen3_32b", 32, False), ("qwen3_32b", 32, True)])
-def test_many_requests_decode_together_at_model_sizes(sized, name, live, copies):
-    """8 to 64 requests decoding in one step at the models' layer sizes: the products with that many
-    rows (own kernel on tile-major weights: whole result, gated, K cut into planes; without the
-    copies the few-row kernel up to 16 rows and the vendor library beyond), decode attention over
-    many sequences. Prompts in three steps, then six steps with a token of every request, against
+@pytest.mark.parametrize("name,live", [("qwen3_4b", 12), ("qwen3_4b", 20), ("qwen3_4b", 40), ("qwen3_4b", 64),
+                                       ("qwen3_8b", 33), ("qwen3_32b", 8), ("qwen3_32b", 32), ("qwen3_32b", 100)])
+def test_many_requests_decode_together_at_model_sizes(sized, name, live):
+    """8 to 100 requests decoding in one step at the models' layer sizes: the products with that
+    many rows (the few-row kernel, the kernel that shares activations: whole result, gated, K cut
+    into planes; the vendor library beyond 64 or 128 rows), decode attention over many sequences. Prompts in three steps, then six steps with a token of every request, against
     the plain implementation of each request alone."""
     cfg, folder = sized[name]
     lengths = [9 + (5 * i) % 23 for i in range(live)]
@@ -143,8 +137,7 @@ def test_many_requests_decode_together_at_model_sizes(sized, name, live, copies)
         steps.append({"entries": [{"id": r, "tokens": reqs[r][len(reqs[r]) - d: len(reqs[r]) - d + 1], "want": [0]}
                                   for r in rids], "end": rids if d == 1 else []})
     steps = traces._number(steps)
-    loaded = load_sized(folder, steps, "bfloat16", copies=copies, max_seqs=live, pages=live * 3, budget=1024)
-    assert bool(loaded.runner.ops._tiled) == copies
+    loaded = load_sized(folder, steps, "bfloat16", max_seqs=live, pages=live * 3, budget=1024)
     got = traces.replay(loaded, steps)
     assert len(got) == live * (decode + 1)
     check_rounding_noise(got, {k: want_all[k] for k in got})
@@ -232,9 +225,8 @@ def test_model_sized_decode_graph_equals_eager(sized):
     traces.compare_logprobs([x for lp in graph_logprobs for x in lp], [x for lp in logprobs for x in lp], std)
 
 
-@pytest.mark.parametrize("name,dtype,copies", [("qwen3_4b", "bfloat16", True), ("qwen3_4b", "float32", True),
-                                               ("qwen3_32b", "bfloat16", False)])
-def test_the_2048_token_prompt_the_measurement_times(sized, name, dtype, copies):
+@pytest.mark.parametrize("name,dtype", [("qwen3_4b", "bfloat16"), ("qwen3_4b", "float32"), ("qwen3_32b", "bfloat16")])
+def test_the_2048_token_prompt_the_measurement_times(sized, name, dtype):
     """One 2,048-token prompt in one step, the step whose time is reported as prefill throughput:
     the vendor products at 2,048 rows, the prompt attention through LDS with 128 (256 at the 32B
     sizes) row tiles and their work list, the wide q/k kernel. Logits at every 16th position and
@@ -243,7 +235,7 @@ def test_the_2048_token_prompt_the_measurement_times(sized, name, dtype, copies)
     wanted = sorted(set(range(0, 2048, 16)) | set(range(2040, 2048)))
     reqs, want = sized.plain_logits(name, [2048], seed=44, positions={"r0": wanted})
     steps = [{"step": 0, "entries": [{"id": "r0", "tokens": reqs["r0"], "want": wanted}], "end": ["r0"]}]
-    got = traces.replay(load_sized(folder, steps, dtype, copies=copies, max_seqs=1), steps)
+    got = traces.replay(load_sized(folder, steps, dtype, max_seqs=1), steps)
     if dtype == "float32":
         traces.compare(got, want, **TOL_F32)
     else:

@@ -231,7 +231,7 @@ def register_toy():
             return decls
 
         def load(self, fetch):
-            self.router = fetch.matrix(self._name("router"), linear=False)
+            self.router = fetch.matrix(self._name("router"))
             for e in range(self.e):
                 base = f"{self._name('expert')}.{e}"
                 self.gate_up.append(fetch.fused([f"{base}.gate", f"{base}.up"], dim=0))
