@@ -679,22 +679,35 @@ static int launch_mid_rows(const bf16_t* a, const bf16_t* w, void* c, int out_dt
   return 0;
 }
 
-// Configurations as timed for the shapes of the 4B and 8B models at 32 and 64 rows, each on the
-// weight matrices of 36 layers in turn (one matrix over and over stays in the memory-side cache
-// and flatters every configuration, the small products most): K groups of two waves with one tile
-// each where the result is wanted whole (three groups from 33 rows on, two below); one group of
-// three waves, a gate and an up tile each, for the gated form; one group of three waves with two
-// tiles each where K is cut over blocks; eight tiles on the staged activations for the
-// vocabulary head. The whole result of an ungated product: up to 64 rows only. Beyond, every
+// Configurations from timing 42 of them per form (1 to 4 K groups, 1 to 8 waves a group, 1 or 2
+// tiles a wave, chunks of 4 to 12 k-steps) on the shapes of the 4B and 8B models at 32, 64 and
+// 128 rows, each on the weight matrices of 36 layers in turn (one matrix over and over stays in
+// the memory-side cache and flatters every configuration, the small products most). Gated: one
+// group of three waves, a gate and an up tile each (20.7, 23.6 and 33.4 us at the 4B size). K cut
+// over blocks: one group whose waves have eight tiles between them, as four waves with two tiles
+// each and chunks of eight k-steps, or, where K is a multiple of 2,048 (the rows of a wave's two
+// tiles then start in the same memory channels) and from 65 rows on (LDS), as eight waves with
+// one tile each and chunks of four (the 8B down projection at 64 rows 19.2 us against 20.5).
+// The whole result: K groups of two waves with one tile each, two groups with chunks of eight,
+// or three with chunks of four where K is a multiple of 2,048; up to 64 rows only: beyond, every
 // block would have to fetch more activations than weights, and the vendor library is faster.
+// Very many tiles (the vocabulary head): eight tiles on the staged activations.
 template <int MB>
 static int mid_rows(const bf16_t* a, const bf16_t* w, void* c, int out_dtype, int M, int N, int K, int gated,
                     hipStream_t st, int k_parts) {
   if (gated) return launch_mid_rows<MB, 1, 3, 1, 6, true>(a, w, c, out_dtype, M, N, K, st, 1);
-  if (k_parts > 1) return launch_mid_rows<MB, 1, 3, 2, 6, false>(a, w, c, out_dtype, M, N, K, st, k_parts);
+  if (k_parts > 1) {
+    if constexpr (MB % 2 == 0) {
+      if (MB > 4 || K % 2048 == 0) return launch_mid_rows<MB, 1, 8, 1, 4, false>(a, w, c, out_dtype, M, N, K, st, k_parts);
+    } else {
+      if (K % 2048 == 0) return launch_mid_rows<MB, 1, 4, 1, 4, false>(a, w, c, out_dtype, M, N, K, st, k_parts);
+    }
+    if constexpr (MB <= 4) return launch_mid_rows<MB, 1, 4, 2, 8, false>(a, w, c, out_dtype, M, N, K, st, k_parts);
+  }
   if constexpr (MB <= 4) {
     if (N >= 32768) return launch_mid_rows<MB, 1, 4, 2, 8, false>(a, w, c, out_dtype, M, N, K, st, 1);
-    return launch_mid_rows<MB, (MB <= 2 ? 2 : 3), 2, 1, 4, false>(a, w, c, out_dtype, M, N, K, st, 1);
+    if (K % 2048 == 0) return launch_mid_rows<MB, 3, 2, 1, 4, false>(a, w, c, out_dtype, M, N, K, st, 1);
+    return launch_mid_rows<MB, 2, 2, 1, 8, false>(a, w, c, out_dtype, M, N, K, st, 1);
   }
   return qrt_fail("gemm_bf16: above 64 rows only the gated form and products cut along K have a kernel of their own (M=%d)", M);
 }

@@ -339,7 +339,7 @@ class HipOps:
     def choose_k_parts(n: int, k: int, m: int = 1, shared: bool | None = None) -> int:
         """The few-row kernel: cut K when there are fewer row tiles than about two per compute
         unit and K is long. The kernel that shares activations (``shared``; by default from 17
-        rows on): a block takes up to six row tiles, and K is cut until there are about as
+        rows on): a block takes up to eight row tiles, and K is cut until there are about as
         many blocks as compute units, each part keeping 12 k-steps or more."""
         tiles = n // 16
         if shared is None:
@@ -353,7 +353,7 @@ class HipOps:
             # against 6.8, 8.9 and 18.3 in eight; the down projection 10.6 and 40.6 us in eight
             # against 12.0 and 43.6 in four at the 4B and 32B sizes, level at the 8B size)
             return 4 if k <= 8192 else 8
-        blocks = (tiles + 5) // 6
+        blocks = (tiles + 7) // 8
         return max(1, min(8, 256 // blocks, (k // 32) // 12))
 
 
