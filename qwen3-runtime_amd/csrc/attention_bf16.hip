@@ -80,6 +80,14 @@ struct AttnTileArgs {
   const float* rope;       // [T, D]: cosines of the D / 2 angles, then their sines; null: no rotation
   const int* slots;        // [T]: place of the token in the cache, page * page_size + offset
   float eps;
+  // Decoding over sequences of very different lengths: instead of num_splits equal parts of every
+  // sequence, pieces of split_blocks 32-key blocks, as many as a sequence has (at most num_splits),
+  // listed in `items` as (sequence, piece), whole pieces first and the sequences' last, shorter
+  // pieces after them, then (-1, 0) up to max_items. The launch is (key head, item): blocks of
+  // equal work, the heavy ones next to each other in launch order, which spreads them evenly over
+  // the compute units. qrt_attention_work_list fills the list from the step's lengths.
+  int split_blocks, max_items;
+  int* items;              // [max_items][2] or null
 };
 
 constexpr int D = QRT_HEAD_DIM;
@@ -820,8 +828,10 @@ __device__ __forceinline__ void merge_few(const float* __restrict__ part_o, cons
       if (s < num_splits) {
         const float w = exp2f(ls[s] - mx);
         wsum += w;
-        acc[0] += w * pv[0][s];
-        acc[1] += w * pv[1][s];
+        if (w > 0.f) {  // the part of an empty split was never written
+          acc[0] += w * pv[0][s];
+          acc[1] += w * pv[1][s];
+        }
       }
     }
   }
@@ -852,7 +862,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
       for (int s = 0; s < num_splits; ++s) {
         const float w = exp2f(lse[s] - mx);
         wsum += w;
-        acc += w * po[(size_t)s * D];
+        if (w > 0.f) acc += w * po[(size_t)s * D];
       }
     }
     out[row * D + d] = (bf16_t)(wsum > 0.f ? acc / wsum : 0.f);
@@ -873,6 +883,53 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
 // write-through atomic stores in place of the fence it costs what the second launch
 // costs.)
 constexpr int DW = 4;
+
+// The 32-key blocks of the cache that a tile of the decode kernel walks: [begin, end). `fused`:
+// the cache holds the keys before the tile's one token (which the kernel adds from registers).
+__device__ __forceinline__ void decode_key_blocks(int kv_len, int q_len, int window, bool fused, int& begin, int& end) {
+  const int own = fused ? 1 : 0;
+  const int first_pos = kv_len - q_len;
+  const int pos_max = first_pos + max(q_len, 1) - 1 - own;
+  const int lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+  const bool any_cached = !fused || (pos_max >= lo && window != 1);
+  begin = lo >> 5;
+  end = any_cached ? (pos_max >> 5) + 1 : begin;
+}
+
+// The work list of a decode launch in pieces (AttnTileArgs::items). One block; up to LIST_TILES
+// sequences. Every sequence has at least one piece (its last piece also takes the token's own key
+// in the fused form), at most ceil(blocks / split_blocks).
+constexpr int LIST_TILES = 1024;
+__global__ __launch_bounds__(256) void attention_work_list_kernel(AttnTileArgs a, int fused) {
+  __shared__ int whole[LIST_TILES + 1], rest[LIST_TILES + 1];  // pieces of each tile, then where they begin
+  for (int t = threadIdx.x; t < a.num_tiles; t += blockDim.x) {
+    const int seq = a.tile_seq ? a.tile_seq[t] : t;
+    int begin, end;
+    decode_key_blocks(a.kv_lens[seq], a.cu_q[seq + 1] - a.cu_q[seq], a.window, fused != 0, begin, end);
+    const int blocks = end - begin;
+    whole[t] = blocks / a.split_blocks;
+    rest[t] = blocks % a.split_blocks != 0 || blocks == 0 ? 1 : 0;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int t = 0; t < a.num_tiles; ++t) { const int n = whole[t]; whole[t] = at; at += n; }
+    whole[a.num_tiles] = at;
+    for (int t = 0; t < a.num_tiles; ++t) { const int n = rest[t]; rest[t] = at; at += n; }
+    rest[a.num_tiles] = at;
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < a.num_tiles; t += blockDim.x) {
+    const int seq = a.tile_seq ? a.tile_seq[t] : t;
+    const int n_whole = whole[t + 1] - whole[t];
+    for (int p = 0; p < n_whole; ++p) {
+      const int at = whole[t] + p;
+      if (at < a.max_items) { a.items[2 * at] = seq; a.items[2 * at + 1] = p; }
+    }
+    if (rest[t + 1] > rest[t] && rest[t] < a.max_items) { a.items[2 * rest[t]] = seq; a.items[2 * rest[t] + 1] = n_whole; }
+  }
+  for (int i = rest[a.num_tiles] + threadIdx.x; i < a.max_items; i += blockDim.x) { a.items[2 * i] = -1; a.items[2 * i + 1] = 0; }
+}
 
 __device__ __forceinline__ void block_compute(KvBlock& blk, const bf16x8_t* qreg, bf16x8_t qtail, int base, int lo,
                                               int pos_min, int pos_max, int quad, bool row_valid, int qpos,
@@ -962,8 +1019,17 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
   // every sequence is one tile here, so without a list the block's number is the sequence's: one
   // dependent load less before the first key arrives. A list names the sequences of a launch
   // that covers only some of the step's.
-  const int seq = a.tile_seq ? a.tile_seq[blockIdx.x] : blockIdx.x;
-  const int kvh = blockIdx.y, split = blockIdx.z;
+  int seq, kvh, split;
+  if (a.items) {  // pieces from the work list: (key head, item)
+    seq = a.items[2 * blockIdx.y];
+    if (seq < 0) return;  // past the end of the list
+    split = a.items[2 * blockIdx.y + 1];
+    kvh = blockIdx.x;
+  } else {
+    seq = a.tile_seq ? a.tile_seq[blockIdx.x] : blockIdx.x;
+    kvh = blockIdx.y;
+    split = blockIdx.z;
+  }
   const int g = a.nq / a.nkv;
   const int q_begin = a.cu_q[seq];
   const int q_len = a.cu_q[seq + 1] - q_begin;
@@ -990,9 +1056,11 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
   const int qpos_c = qpos - own;
   const int pos_min = first_pos - own, pos_max = first_pos + (max(n_rows, 1) - 1) / g - own;
   const int lo = a.window > 0 ? max(0, first_pos - a.window + 1) : 0;
-  const bool any_cached = !FUSED || (pos_max >= lo && a.window != 1);
-  const int blk_begin = lo >> 5, blk_end = any_cached ? (pos_max >> 5) + 1 : blk_begin;
-  const int per = (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
+  int blk_begin, blk_end;
+  decode_key_blocks(kv_len, q_len, a.window, FUSED, blk_begin, blk_end);
+  // equal parts of the sequence's blocks, or pieces of a fixed length, as many as it has
+  const int per = a.items ? a.split_blocks : (blk_end - blk_begin + a.num_splits - 1) / a.num_splits;
+  const int last_split = a.items ? max(1, (blk_end - blk_begin + per - 1) / per) - 1 : (int)gridDim.z - 1;
   const int b0 = blk_begin + split * per;
   const int b1 = min(blk_end, b0 + per);
   int b = b0 + wave;
@@ -1007,7 +1075,7 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
     const bf16_t* raw = a.qkv + (size_t)q_begin * a.qkv_stride;
     const float* rope = a.rope ? a.rope + (size_t)q_begin * D : nullptr;
     head_as_operand(raw + (size_t)head * D, a.q_weight, rope, a.eps, quad, qreg);
-    const bool at_end = split == (int)gridDim.z - 1;
+    const bool at_end = split == last_split;
     const bool adds_own = at_end && wave == DW - 1, stores_own = at_end && wave == (2 * DW - 2) % DW;
     if (adds_own || stores_own) {  // uniform over the wave
       const bf16_t* kraw = raw + ((size_t)a.nq + kvh) * D;
@@ -1121,6 +1189,30 @@ __global__ __launch_bounds__(64 * DW, D <= 128 ? 2 : 1) void attention_bf16_deco
       if (d == 0) a.part_lse[row_index * a.num_splits + split] = den > 0.f ? mm + log2f(den) : -INFINITY;
     }
   }
+  // the pieces this sequence does not have count as empty splits (their parts are never read)
+  if (a.items && split == 0) {
+    const int missing = a.num_splits - 1 - last_split;
+    for (int idx = threadIdx.x; idx < n_rows * missing; idx += 64 * DW) {
+      const int row = idx % n_rows, s = last_split + 1 + idx / n_rows;
+      const int rt = row / g, rh = row - rt * g;
+      a.part_lse[(tile_row0 + (size_t)rt * a.nq + kvh * g + rh) * a.num_splits + s] = -INFINITY;
+    }
+  }
+}
+
+// Fills args->items for a decode launch in pieces of args->split_blocks blocks: needs cu_q,
+// kv_lens, tile_seq (or null), num_tiles <= 1024, window, max_items >= the pieces there can be
+// (num_tiles * num_splits will do). `fused` as the launch: the tokens' own keys come from the
+// product, the cache holds the keys before them.
+extern "C" int qrt_attention_work_list(const AttnTileArgs* args, int fused, hipStream_t stream) {
+  const AttnTileArgs& a = *args;
+  QRT_CHECK(a.items && a.split_blocks > 0 && a.num_tiles >= 0 && a.num_tiles <= LIST_TILES && a.max_items >= a.num_tiles,
+            "attention work list: %d sequences (at most %d), %d items, pieces of %d blocks", a.num_tiles, LIST_TILES,
+            a.max_items, a.split_blocks);
+  if (a.max_items == 0) return 0;
+  attention_work_list_kernel<<<1, 256, 0, stream>>>(a, fused);
+  QRT_LAUNCH_CHECK("attention_work_list");
+  return 0;
 }
 
 // every listed sequence at most 16 rows (q_len * g <= 16) and D <= 256; num_tiles = number of
@@ -1135,9 +1227,14 @@ extern "C" int qrt_attention_bf16_decode(const AttnTileArgs* args, int num_rows_
   QRT_CHECK(a.num_splits >= 1 && a.num_splits <= 65535 && a.nkv <= 65535, "attention: bad split or head count");
   QRT_CHECK(a.num_splits == 1 || (a.part_o && a.part_lse), "attention: split run without scratch");
   QRT_CHECK(a.table_width > 0 && a.window >= 0, "attention: bad table width or window");
+  QRT_CHECK(a.items ? a.split_blocks > 0 && a.max_items >= a.num_tiles && a.max_items <= 65535
+                    : a.split_blocks == 0,
+            "attention (decode): pieces of %d blocks with a list of %d items for %d sequences", a.split_blocks,
+            a.max_items, a.num_tiles);
   if (a.num_tiles == 0) return 0;
   const bool p2 = (a.page_size & (a.page_size - 1)) == 0;  // shifts instead of divisions
   dim3 grid(a.num_tiles, a.nkv, a.num_splits), block(64 * DW);
+  if (a.items) grid = dim3(a.nkv, a.max_items, 1);
   constexpr size_t smem = (size_t)(2 * DW * 16 + DW * 16 * D) * sizeof(float);
   if (smem > 64 * 1024) {  // head size 256: a little more LDS than a block gets without asking
     static bool allowed = false;  // once: not again inside every stream capture

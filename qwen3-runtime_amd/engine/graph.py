@@ -1,6 +1,7 @@
 """Pure-decode steps replayed from captured HIP graphs.
 
-A graph is captured per (batch size, bucket of the longest context). Its
+A graph is captured per (batch size, bucket of the longest context, whether the
+contexts are of very unequal lengths: the attention kernel then cuts them another way). Its
 kernels read the step's arrays (token ids, positions, lengths, block tables,
 slots) from one static device buffer; a replay fills that buffer with one copy
 and launches the whole step at once, which removes the per-kernel launch cost
@@ -27,17 +28,17 @@ MIN_BUCKET = 512
 
 class DecodeGraph:
     @staticmethod
-    def key_for(batch: int, max_kv: int, all_want: bool):
+    def key_for(batch: int, max_kv: int, all_want: bool, unequal: bool = False):
         if not all_want:
             return None
         bucket = MIN_BUCKET
         while bucket < max_kv:
             bucket *= 2
-        return (batch, bucket)
+        return (batch, bucket, bool(unequal))
 
     def __init__(self, runner, key):
         self.runner = runner
-        self.batch, self.bucket = key
+        self.batch, self.bucket, self.unequal = key
         cache = runner.cache
         self.width = max(1, -(-self.bucket // cache.page_size))
         self.graph: torch.cuda.CUDAGraph | None = None
@@ -212,7 +213,11 @@ class DecodeGraph:
                 self.views_dev = self._views()
                 packed.kv_lens = [self.bucket] * self.batch  # launch shapes are those of the bucket
                 self.ctx = runner._context(packed, self.views_dev)
-                # the bucket's length, not the batch's, now fixes every launch shape (key splits too)
+                # the bucket's length, not the batch's, now fixes every launch shape (key splits too);
+                # where the lengths are very unequal the attention kernel is told them as they are
+                # now, to choose the length of its pieces by
+                if self.unequal:
+                    self.ctx.scratch["attn_lens"] = [runner.cache.length(e.request_id) + 1 for e in entries]
                 self.cache_views = [
                     None if st.cache is None else runner.cache.view(st.cache, self.ctx.groups, st.writes_cache)
                     for st in runner.model.plan.order

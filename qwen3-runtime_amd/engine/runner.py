@@ -170,8 +170,12 @@ class ModelRunner:
     def _step_graph(self, entries: Sequence[StepEntry]):
         from .graph import DecodeGraph
 
-        max_kv = max(self.cache.length(e.request_id) + 1 for e in entries)
-        key = DecodeGraph.key_for(len(entries), max_kv, all(len(e.want) == 1 for e in entries))
+        lens = [self.cache.length(e.request_id) + 1 for e in entries]
+        max_kv = max(lens)
+        # contexts of very unequal lengths: the ops may cut them another way, which a capture freezes
+        unequal = getattr(self.ops, "decode_in_pieces", None)
+        key = DecodeGraph.key_for(len(entries), max_kv, all(len(e.want) == 1 for e in entries),
+                                  unequal is not None and unequal(lens))
         if key is None:
             packed = pack_step(entries, self.cache, self.vocab_size)
             dev = self._upload(packed)

@@ -66,7 +66,8 @@ class _AttnTileArgs(Structure):
         ("scale_log2", c_float), ("row_tiles", c_int), ("use_lds", c_int),
         ("merge_tokens", c_void_p), ("num_merge_tokens", c_int),
         ("qkv", c_void_p), ("qkv_stride", c_long), ("q_weight", c_void_p), ("k_weight", c_void_p),
-        ("rope", c_void_p), ("slots", c_void_p), ("eps", c_float),
+        ("rope", c_void_p), ("slots", c_void_p), ("eps", c_float), ("split_blocks", c_int),
+        ("max_items", c_int), ("items", c_void_p),
     ]
 
 
@@ -635,6 +636,31 @@ class HipOps:
         blocks = (max_kv + 31) // 32
         return max(1, min((256 + work - 1) // work, blocks // 8, 64))
 
+    # decoding over unequal lengths: from this ratio of the longest to the mean length on, pieces
+    decode_piece_ratio = 1.3
+
+    def decode_in_pieces(self, kv_lens) -> bool:
+        """Whether a decode launch over sequences of these lengths cuts their keys into pieces
+        of one length (as many per sequence as it has) instead of every sequence into equally
+        many parts."""
+        n, total = len(kv_lens), sum(kv_lens)
+        return n >= 2 and max(kv_lens) * n > self.decode_piece_ratio * total and max(kv_lens) > 1024
+
+    def choose_decode_piece(self, kv_lens, nkv: int):
+        """Keys per piece for such a launch (a multiple of 32), or None. Equal parts of every
+        sequence make blocks whose work is the sequence's length: with 56 sequences of 300 keys
+        and 8 of 8,000 the launch takes 231 us where the two kinds alone take 18 and 48, and more
+        parts do not help, because the blocks reach the compute units in launch order, round
+        robin, and heavy blocks a fixed stride apart land on the same few. Pieces of one length,
+        whole ones first in the list: about 1,536 blocks in all, no piece under 512 keys (a block
+        costs some 8 us before its first key arrives) and no sequence in more than 16 (the merge
+        reads every piece's part: 8 sequences of 1,000 to 30,000 keys 83 us in pieces of 2,048
+        against 113 in pieces of 544)."""
+        if not self.decode_in_pieces(kv_lens):
+            return None
+        piece = max(512, -(-sum(kv_lens) * nkv // 1536), -(-max(kv_lens) // 16))
+        return -(-piece // 32) * 32
+
     # mixed steps: sequences with few rows leave the prompt kernel when their context is this long
     split_launch_min_kv = 1024
 
@@ -704,6 +730,21 @@ class HipOps:
         splits = ctx.scratch.get("attn_splits") or (
             self.choose_decode_splits(n_tiles, nkv, max_kv) if decode else self.choose_splits(n_tiles, nkv, max_kv))
         a = _AttnTileArgs()
+        piece = None
+        if decode and n_tiles <= 1024:
+            piece = ctx.scratch.get("attn_piece")  # keys per piece, a multiple of 32: asked for outright
+            if piece is None and "attn_splits" not in ctx.scratch:
+                # the lengths as they are; a capture sees its bucket's instead and is told them beside
+                piece = self.choose_decode_piece(ctx.scratch.get("attn_lens") or kv_lens, nkv)
+        if piece:
+            a.split_blocks = piece // 32
+            # 32-key blocks a sequence of this launch can have: all its keys, or those of its
+            # window, which may begin and end inside a block
+            span = (max_kv + 31) // 32 if not window else (min(max_kv, window + 32) + 31) // 32 + 1
+            splits = max(1, -(-span // a.split_blocks))
+            if n_tiles * splits > 65535:
+                piece, a.split_blocks = None, 0
+                splits = self.choose_decode_splits(n_tiles, nkv, max_kv)
         a.out, a.k_cache, a.v_cache = out.data_ptr(), cache.k.data_ptr(), cache.v.data_ptr()
         if own is None:
             a.q = q.data_ptr()
@@ -728,6 +769,17 @@ class HipOps:
             part_o = torch.empty((ctx.num_tokens * nq * splits, d), dtype=torch.float32, device=out.device)
             part_lse = torch.empty((ctx.num_tokens * nq * splits,), dtype=torch.float32, device=out.device)
             a.part_o, a.part_lse = part_o.data_ptr(), part_lse.data_ptr()
+        if piece:
+            # the list of (sequence, piece): from the step's lengths on the device, once per pass
+            a.max_items = n_tiles * splits
+            list_key = ("attn_items", key, window, own is not None, piece, a.max_items)
+            items = ctx.per_pass.get(list_key)
+            if items is None:
+                items = torch.empty((a.max_items, 2), dtype=torch.int32, device=out.device)
+                a.items = items.data_ptr()
+                self._check(lib, lib.qrt_attention_work_list(byref(a), c_int(own is not None), _stream()))
+                ctx.per_pass[list_key] = items
+            a.items = items.data_ptr()
         if decode:
             self._check(lib, lib.qrt_attention_bf16_decode(byref(a), c_int(ctx.num_tokens * nq), _stream()))
         else:

@@ -588,6 +588,16 @@ def test_decode_attention_with_the_tokens_own_key_from_the_product(ops, nq, nkv,
         cache.v.copy_(before_v)
         ctx.scratch["attn_splits"] = splits
         close(ops.decode_attention(qkv, cache, ctx, nq, nkv, d, scale, window, qw, kw, 1e-6, inv), want, 2e-2, 2e-2)
+    # ... and into pieces of one length, listed sequence by sequence (one block of keys each, so
+    # that the longest has 66 and the shortest none but the token itself; three blocks; sixteen)
+    del ctx.scratch["attn_splits"]
+    for piece in (32, 96, 512):
+        cache.k.copy_(before_k)
+        cache.v.copy_(before_v)
+        ctx.scratch["attn_piece"] = piece
+        ctx.per_pass.clear()
+        close(ops.decode_attention(qkv, cache, ctx, nq, nkv, d, scale, window, qw, kw, 1e-6, inv), want, 2e-2, 2e-2)
+        assert torch.equal(cache.k[~changed_k], before_k[~changed_k]) and torch.equal(cache.v[~changed_v], before_v[~changed_v])
 
 
 @pytest.mark.parametrize("nq,nkv,d,ps,window", [(32, 8, 128, 16, None), (8, 2, 64, 8, None), (8, 2, 64, 16, 40)])
@@ -846,6 +856,55 @@ def test_decode_attention_many_sequences_and_repeated_launches(ops):
             ctx.scratch["attn_splits"] = splits
         got = ops.paged_attention(q, cache, ctx, nq, nkv, d, 0.088, None)
         close(got, want, 2e-2, 2e-2)
+
+
+@pytest.mark.parametrize("seqs,nq,nkv,d,ps,window", [
+    ([(1, n) for n in (300, 5000, 1, 33, 2048, 700, 64, 4097)], 8, 2, 128, 16, None),
+    ([(1, 300)] * 20 + [(1, 6000)] * 3, 32, 8, 128, 16, None),           # few long ones among many short
+    ([(2, 1500), (4, 40), (1, 3000), (3, 3)], 4, 1, 64, 8, None),        # tiles of several tokens
+    ([(1, 2500), (1, 90), (1, 700)], 6, 2, 32, 24, 200),                 # a window, pages of 24
+    ([(1, 1100), (1, 20)], 2, 2, 256, 16, None),
+])
+def test_decode_attention_in_pieces_of_one_length(ops, seqs, nq, nkv, d, ps, window):
+    """Sequences of very unequal lengths: the decode kernel walks a list of (sequence, piece), the
+    pieces all of one length (the choice by the lengths, and lengths asked for outright: one
+    block of 32 keys, so that the merge has up to 157 parts, and up to more than the longest
+    sequence), unwritten places of the cache full of NaN. The list is made on the device from the
+    step's lengths: also after the lengths have changed under the same context, as they do under
+    a captured graph."""
+    q, cache, ctx = build_attention_case(seqs, nq, nkv, d, ps, torch.bfloat16, seed=8, window=window, poison=True)
+    scale = 1.0 / math.sqrt(d)
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, scale, window)
+    kv_lens = [kv for _, kv in seqs]
+    assert ops.decode_in_pieces(kv_lens) and ops.choose_decode_piece(kv_lens, nkv) % 32 == 0
+    for piece in (None, 32, 512, 8192):
+        ctx.scratch.pop("attn_piece", None)
+        if piece:
+            ctx.scratch["attn_piece"] = piece
+        ctx.per_pass.clear()
+        close(ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, window), want, 2e-2, 2e-2)
+    # the same launch shapes over shorter sequences: every length cut to a third on the device only,
+    # the host's view (what a captured launch was shaped for) unchanged
+    ctx.scratch["attn_piece"] = 512
+    short = [(q_len, max(q_len, kv // 3)) for q_len, kv in seqs]
+    ctx.kv_lens.copy_(torch.tensor([kv for _, kv in short], dtype=torch.int32))
+    want = R.paged_attention(q, cache.k, cache.v, ctx.cu_q.cpu(), ctx.kv_lens.cpu(), cache.group.block_table,
+                             ps, nq, nkv, d, scale, window)
+    ctx.per_pass.clear()
+    close(ops.paged_attention(q, cache, ctx, nq, nkv, d, scale, window), want, 2e-2, 2e-2)
+
+
+def test_which_decode_launches_go_in_pieces(ops):
+    """Equal lengths keep equal parts; very unequal ones get pieces of at least 512 keys, at most 16
+    for the longest sequence, about 1,536 blocks in all."""
+    assert not ops.decode_in_pieces([2100] * 64) and not ops.decode_in_pieces([2048]) and not ops.decode_in_pieces([900, 100])
+    assert ops.decode_in_pieces([300] * 56 + [8000] * 8) and ops.decode_in_pieces([500, 16000])
+    assert ops.choose_decode_piece([2100] * 64, 8) is None
+    assert ops.choose_decode_piece([300] * 56 + [8000] * 8, 8) == 512
+    assert ops.choose_decode_piece([500, 16000], 8) == 1024
+    assert ops.choose_decode_piece([1000, 30000] * 4, 8) == 1888
+    assert ops.choose_decode_piece(list(range(128, 4352, 33)), 8) == 1504
 
 
 @pytest.mark.parametrize("seqs,nq,nkv,d,ps", [([(9, 50)], 3, 3, 80, 16), ([(2, 300), (1, 50)], 5, 1, 48, 8),

@@ -188,6 +188,37 @@ def test_six_layers_deep(sized, dtype):
         check_rounding_noise(got, want)
 
 
+@pytest.mark.parametrize("graph", [False, True])
+def test_contexts_of_very_unequal_lengths_decode_in_pieces(sized, graph, monkeypatch):
+    """Requests of 1,600, 45 and 260 tokens decode together, eagerly and from replayed graphs: the
+    decode attention then cuts the keys into pieces of one length from a list made on the device
+    at every step (a captured graph is told the lengths at its capture and shaped for its bucket;
+    the lengths go on growing under it). Logits of the last eight tokens of each request against
+    the plain implementation."""
+    from qwen3_runtime_amd.ops.hip import HipOps
+
+    cfg, folder = sized["qwen3_4b"]
+    reqs, want = sized.plain_logits("qwen3_4b", [1600, 45, 260], seed=52)
+    rids, decode = list(reqs), 8
+    steps = [{"entries": [{"id": r, "tokens": reqs[r][:-decode], "want": [len(reqs[r]) - decode - 1]}], "end": []}
+             for r in rids]
+    for d in range(decode, 0, -1):
+        steps.append({"entries": [{"id": r, "tokens": reqs[r][len(reqs[r]) - d: len(reqs[r]) - d + 1], "want": [0]}
+                                  for r in rids], "end": rids if d == 1 else []})
+    steps = traces._number(steps)
+    pieces = []
+    inner = HipOps.choose_decode_piece
+    monkeypatch.setattr(HipOps, "choose_decode_piece",
+                        lambda self, lens, nkv: (pieces.append(inner(self, lens, nkv)), pieces[-1])[1])
+    loaded = load_sized(folder, steps, "bfloat16", graph=graph)
+    got = traces.replay(loaded, steps)
+    assert pieces and all(p == 512 for p in pieces), "the decode steps were cut into pieces"
+    if graph:
+        assert any(key[2] for key in loaded.runner._graphs), "a graph for unequal lengths was captured and replayed"
+    assert len(got) == 3 * (decode + 1)
+    check_rounding_noise(got, {k: want[k] for k in got})
+
+
 def test_model_sized_decode_graph_equals_eager(sized):
     """Three requests at the 4B layer sizes, decoded eagerly and then from replayed HIP graphs that
     are fed the eager tokens: at every token the graph's log-probability of it is the eager one up
