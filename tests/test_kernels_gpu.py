@@ -863,7 +863,7 @@ def test_decode_attention_many_sequences_and_repeated_launches(ops):
     ([(1, 300)] * 20 + [(1, 6000)] * 3, 32, 8, 128, 16, None),           # few long ones among many short
     ([(2, 1500), (4, 40), (1, 3000), (3, 3)], 4, 1, 64, 8, None),        # tiles of several tokens
     ([(1, 2500), (1, 90), (1, 700)], 6, 2, 32, 24, 200),                 # a window, pages of 24
-    ([(1, 1100), (1, 20)], 2, 2, 256, 16, None),
+    ([(1, 2100), (1, 20)], 2, 2, 256, 16, None),
 ])
 def test_decode_attention_in_pieces_of_one_length(ops, seqs, nq, nkv, d, ps, window):
     """Sequences of very unequal lengths: the decode kernel walks a list of (sequence, piece), the
@@ -898,7 +898,8 @@ def test_decode_attention_in_pieces_of_one_length(ops, seqs, nq, nkv, d, ps, win
 def test_which_decode_launches_go_in_pieces(ops):
     """Equal lengths keep equal parts; very unequal ones get pieces of at least 512 keys, at most 16
     for the longest sequence, about 1,536 blocks in all."""
-    assert not ops.decode_in_pieces([2100] * 64) and not ops.decode_in_pieces([2048]) and not ops.decode_in_pieces([900, 100])
+    assert not ops.decode_in_pieces([2100] * 64) and not ops.decode_in_pieces([2048]) and not ops.decode_in_pieces([1900, 100])
+    assert not ops.decode_in_pieces([2000, 3000, 2500, 2600])
     assert ops.decode_in_pieces([300] * 56 + [8000] * 8) and ops.decode_in_pieces([500, 16000])
     assert ops.choose_decode_piece([2100] * 64, 8) is None
     assert ops.choose_decode_piece([300] * 56 + [8000] * 8, 8) == 512

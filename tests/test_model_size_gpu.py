@@ -190,7 +190,7 @@ def test_six_layers_deep(sized, dtype):
 
 @pytest.mark.parametrize("graph", [False, True])
 def test_contexts_of_very_unequal_lengths_decode_in_pieces(sized, graph, monkeypatch):
-    """Requests of 1,600, 45 and 260 tokens decode together, eagerly and from replayed graphs: the
+    """Requests of 2,300, 45 and 260 tokens decode together, eagerly and from replayed graphs: the
     decode attention then cuts the keys into pieces of one length from a list made on the device
     at every step (a captured graph is told the lengths at its capture and shaped for its bucket;
     the lengths go on growing under it). Logits of the last eight tokens of each request against
@@ -198,7 +198,7 @@ def test_contexts_of_very_unequal_lengths_decode_in_pieces(sized, graph, monkeyp
     from qwen3_runtime_amd.ops.hip import HipOps
 
     cfg, folder = sized["qwen3_4b"]
-    reqs, want = sized.plain_logits("qwen3_4b", [1600, 45, 260], seed=52)
+    reqs, want = sized.plain_logits("qwen3_4b", [2300, 45, 260], seed=52)
     rids, decode = list(reqs), 8
     steps = [{"entries": [{"id": r, "tokens": reqs[r][:-decode], "want": [len(reqs[r]) - decode - 1]}], "end": []}
              for r in rids]
