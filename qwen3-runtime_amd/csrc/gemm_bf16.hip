@@ -552,6 +552,7 @@ __global__ __launch_bounds__(64 * KW * NWV) void gemm_bf16_mid_rows_kernel(const
   auto run_chunk = [&](int c, auto last) {
     constexpr bool LAST = decltype(last)::value;
     QRT_WAIT_LOADS(PAIRS * WLOADS);  // this wave's share of the activations of chunk c has landed
+    QRT_WAIT_LDS();                  // and its reads of the chunk before are in registers
     QRT_BARRIER();                   // everybody's has, and nobody reads the other buffer any more
     if (!LAST) fetch_activations(c + 1);
     const unsigned char* cur = group_buf + (c & 1) * ABUF;
