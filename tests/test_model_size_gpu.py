@@ -219,8 +219,11 @@ def test_contexts_of_very_unequal_lengths_decode_in_pieces(sized, graph, monkeyp
     check_rounding_noise(got, {k: want[k] for k in got})
 
 
-def test_model_sized_decode_graph_equals_eager(sized):
-    """Three requests at the 4B layer sizes, decoded eagerly and then from replayed HIP graphs that
+@pytest.mark.parametrize("lengths", [[70, 20, 5], [2200, 30, 300]])
+def test_model_sized_decode_graph_equals_eager(sized, lengths):
+    """(The second set of lengths is unequal enough for the decode attention to walk pieces from
+    its work list, under graphs whose key says so, with steps launched ahead of their turn.)
+    Three requests at the 4B layer sizes, decoded eagerly and then from replayed HIP graphs that
     are fed the eager tokens: at every token the graph's log-probability of it is the eager one up
     to the rounding of bfloat16. (A graph cuts the keys for the length of its bucket, an eager step
     for the length of the step's longest context, so the partial sums of attention are formed in
@@ -230,17 +233,17 @@ def test_model_sized_decode_graph_equals_eager(sized):
     from qwen3_runtime_amd.llm import LLM
 
     cfg, folder = sized["qwen3_4b"]
-    prompts = list(traces.make_requests(cfg.vocab_size, [70, 20, 5], seed=8).values())
+    prompts = list(traces.make_requests(cfg.vocab_size, lengths, seed=8).values())
 
     def run(graph, forced=None):
-        llm = LLM(str(folder), dtype="bfloat16", max_num_seqs=4, max_num_batched_tokens=64, block_size=16,
-                  num_kv_blocks=64, cuda_graph=graph)
+        llm = LLM(str(folder), dtype="bfloat16", max_num_seqs=4, max_num_batched_tokens=max(64, max(lengths) // 4),
+                  block_size=16, num_kv_blocks=64 + sum(lengths) // 16, cuda_graph=graph)
         eng = llm.engine
         reqs = [eng.request(eng.add_request(p, 24, forced_tokens=None if forced is None else forced[i]))
                 for i, p in enumerate(prompts)]
         while not eng.is_finished():
             eng.step()
-        replayed = bool(eng.runner._graphs)
+        replayed = bool(eng.runner._graphs) and (max(lengths) < 2048 or any(key[2] for key in eng.runner._graphs))
         out = [r.output_tokens for r in reqs], [r.logprobs for r in reqs]
         del llm, eng
         torch.cuda.empty_cache()
@@ -251,7 +254,7 @@ def test_model_sized_decode_graph_equals_eager(sized):
     assert replayed, "no decode step was replayed from a graph"
     assert again == tokens
     # both are bfloat16 with other partial sums: rounding noise in units of the logits' deviation
-    _, want = sized.plain_logits("qwen3_4b", [70, 20, 5], seed=8)
+    _, want = sized.plain_logits("qwen3_4b", lengths, seed=8)
     std = float(torch.stack(list(want.values())).double().std())
     traces.compare_logprobs([x for lp in graph_logprobs for x in lp], [x for lp in logprobs for x in lp], std)
 
