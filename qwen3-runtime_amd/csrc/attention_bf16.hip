@@ -847,9 +847,11 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
   // rows are (token, query head); with a token list the grid walks the listed tokens' rows only
   const size_t row = tokens ? (size_t)tokens[blockIdx.x / nq] * nq + blockIdx.x % nq : blockIdx.x;
   const float* lse = part_lse + row * num_splits;
-  if (num_splits <= 16 && D <= 2 * (int)blockDim.x) {
+  if (num_splits <= 64 && D <= 2 * (int)blockDim.x) {
     if (num_splits <= 8) merge_few<8>(part_o, lse, out, num_splits, row);
-    else merge_few<16>(part_o, lse, out, num_splits, row);
+    else if (num_splits <= 16) merge_few<16>(part_o, lse, out, num_splits, row);
+    else if (num_splits <= 32) merge_few<32>(part_o, lse, out, num_splits, row);
+    else merge_few<64>(part_o, lse, out, num_splits, row);
     return;
   }
   float mx = -INFINITY;

@@ -631,7 +631,9 @@ class HipOps:
 
     @staticmethod
     def choose_decode_splits(num_tiles: int, nkv: int, max_kv: int) -> int:
-        """Decoding: blocks of four waves; about 256 blocks in all, at least 8 key blocks of 32 each."""
+        """Decoding: blocks of four waves; about 256 blocks in all, at least 8 key blocks of 32 each
+        (4 each measured 2 % slower over a batch-1 decode step at 2,048 keys), at most 64 parts
+        (what the merge kernel reads with every load in flight at once)."""
         work = num_tiles * nkv
         blocks = (max_kv + 31) // 32
         return max(1, min((256 + work - 1) // work, blocks // 8, 64))
@@ -656,12 +658,12 @@ class HipOps:
         parts do not help, because the blocks reach the compute units in launch order, round
         robin, and heavy blocks a fixed stride apart land on the same few. Pieces of one length,
         whole ones first in the list: about 1,536 blocks in all, no piece under 512 keys (a block
-        costs some 8 us before its first key arrives) and no sequence in more than 16 (the merge
-        reads every piece's part: 8 sequences of 1,000 to 30,000 keys 83 us in pieces of 2,048
-        against 113 in pieces of 544)."""
+        costs some 8 us before its first key arrives) and no sequence in more than 32 (the merge
+        reads every piece's part, up to 64 with all its loads in flight at once: 8 sequences of
+        1,000 to 30,000 keys 91 us in pieces of 1,024, 96 in pieces of 512, 126 in pieces of 4,096)."""
         if not self.decode_in_pieces(kv_lens):
             return None
-        piece = max(512, -(-sum(kv_lens) * nkv // 1536), -(-max(kv_lens) // 16))
+        piece = max(512, -(-sum(kv_lens) * nkv // 1536), -(-max(kv_lens) // 32))
         return -(-piece // 32) * 32
 
     # mixed steps: sequences with few rows leave the prompt kernel when their context is this long

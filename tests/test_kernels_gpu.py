@@ -896,15 +896,15 @@ def test_decode_attention_in_pieces_of_one_length(ops, seqs, nq, nkv, d, ps, win
 
 
 def test_which_decode_launches_go_in_pieces(ops):
-    """Equal lengths keep equal parts; very unequal ones get pieces of at least 512 keys, at most 16
+    """Equal lengths keep equal parts; very unequal ones get pieces of at least 512 keys, at most 32
     for the longest sequence, about 1,536 blocks in all."""
     assert not ops.decode_in_pieces([2100] * 64) and not ops.decode_in_pieces([2048]) and not ops.decode_in_pieces([1900, 100])
     assert not ops.decode_in_pieces([2000, 3000, 2500, 2600])
     assert ops.decode_in_pieces([300] * 56 + [8000] * 8) and ops.decode_in_pieces([500, 16000])
     assert ops.choose_decode_piece([2100] * 64, 8) is None
     assert ops.choose_decode_piece([300] * 56 + [8000] * 8, 8) == 512
-    assert ops.choose_decode_piece([500, 16000], 8) == 1024
-    assert ops.choose_decode_piece([1000, 30000] * 4, 8) == 1888
+    assert ops.choose_decode_piece([500, 16000], 8) == 512
+    assert ops.choose_decode_piece([1000, 30000] * 4, 8) == 960
     assert ops.choose_decode_piece(list(range(128, 4352, 33)), 8) == 1504
 
 
