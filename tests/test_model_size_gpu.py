@@ -219,6 +219,50 @@ def test_contexts_of_very_unequal_lengths_decode_in_pieces(sized, graph, monkeyp
     check_rounding_noise(got, {k: want[k] for k in got})
 
 
+def test_traffic_of_unequal_lengths_through_the_scheduler_from_graphs(sized):
+    """Eight requests of 30 to 3,500 prompt tokens arrive one after the other at an engine with
+    room for four and a pool that holds the first four prompts and little more; they decode from
+    graphs, steps launched ahead, the attention in equal parts or in pieces as the lengths of the
+    moment say. Every request is fed given tokens, and the engine's log-probability of each (after
+    portions and waiting, beside whichever others were there) has to be the plain
+    implementation's up to rounding noise."""
+    import random
+
+    from plain import qwen3_plain as P
+    from qwen3_runtime_amd.llm import LLM
+
+    cfg, folder = sized["qwen3_4b"]
+    rng = random.Random(4)
+    lengths = [3500, 40, 900, 2600, 30, 300, 3100, 120]
+    prompts = list(traces.make_requests(cfg.vocab_size, lengths, seed=61).values())
+    forced = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(6, 20))] for _ in lengths]
+    arrive = [0, 0, 1, 3, 6, 9, 12, 20]
+    pages = sum(lengths[:4]) // 16 + 6  # the first four prompts and a little: they cannot all grow
+    llm = LLM(str(folder), dtype="bfloat16", max_num_seqs=4, max_num_batched_tokens=1024, block_size=16,
+              num_kv_blocks=pages, cuda_graph=True)
+    eng = llm.engine
+    reqs, step = {}, 0
+    while len(reqs) < len(lengths) or not eng.is_finished():
+        while len(reqs) < len(lengths) and arrive[len(reqs)] <= step:
+            i = len(reqs)
+            reqs[i] = eng.request(eng.add_request(prompts[i], len(forced[i]), forced_tokens=forced[i]))
+        eng.step()
+        eng.cache.check()
+        step += 1
+        assert step < 5000, "the engine makes no progress"
+    keys = list(eng.runner._graphs)
+    assert any(key[2] for key in keys) and eng.cache.num_free_pages == pages
+    assert eng.runner.steps_ahead[1] >= 1, "no step was launched ahead of its turn"
+    cfg_plain, w = P.read_model(folder, device=DEVICE)
+    got_lp, want_lp = [], []
+    for i in range(len(lengths)):
+        assert reqs[i].output_tokens == forced[i]
+        lp, _, std = traces.plain_logprobs(cfg_plain, w, prompts[i], forced[i])
+        got_lp += reqs[i].logprobs
+        want_lp += lp
+    traces.compare_logprobs(got_lp, want_lp, std)
+
+
 @pytest.mark.parametrize("lengths", [[70, 20, 5], [2200, 30, 300]])
 def test_model_sized_decode_graph_equals_eager(sized, lengths):
     """(The second set of lengths is unequal enough for the decode attention to walk pieces from
