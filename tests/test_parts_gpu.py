@@ -625,3 +625,139 @@ def test_a_paged_cache_of_latent_vectors(latent_folder, dtype):
         traces.compare(got, want, atol=5e-5, rtol=5e-5)
     else:
         traces.compare_rounding_noise(got, want)
+
+
+# ------------------------------------------------------------------------------------------------
+# A third toy: a norm and an arrangement of the block of its own, around the framework's attention
+# and feed-forward.
+# ------------------------------------------------------------------------------------------------
+PARALLEL = {"architectures": ["ToyParallelForCausalLM"], "vocab_size": 150, "hidden_size": 64, "head_dim": 16,
+            "heads": 4, "kv_heads": 2, "intermediate_size": 96, "eps": 1e-5, "theta": 20000.0, "max_positions": 256}
+
+
+@pytest.fixture(scope="module")
+def parallel_folder(tmp_path_factory):
+    from qwen3_runtime_amd.parts.base import Block, Norm
+    from qwen3_runtime_amd.parts.plan import CacheSpec, LayerSpec, ModelPlan, PartSpec, RunStep, TensorDecl
+    from qwen3_runtime_amd.registry import (register_architecture, register_part, unregister_architecture,
+                                            unregister_part)
+    from qwen3_runtime_amd.weights import write_model_folder
+
+    @register_part("norm", "toy_centered")
+    class CenteredNorm(Norm):
+        """y = c * rsqrt(mean(c^2) + eps) * w with c = x - mean(x): the mean goes too, unlike RMSNorm.
+        In float32, in torch; it adds what is pending into the residual stream first, as any norm
+        here does (one matrix or several planes), and normalises only the rows asked for."""
+
+        def __init__(self, size, eps, tensors=None):
+            super().__init__(tensors)
+            self.size, self.eps, self.weight = size, eps, None
+
+        def tensor_decls(self):
+            return [TensorDecl(self._name("weight"), (self.size,), init="norm")]
+
+        def load(self, fetch):
+            self.weight = fetch.vector_f32(self._name("weight"))
+
+        def forward(self, ctx, residual, delta=None, rows=None):
+            pending = None if delta is None else (delta.sum(0) if delta.dim() == 3 else delta.float())
+            if rows is None:
+                if pending is not None:
+                    residual.add_(pending)
+                x = residual
+            else:
+                x = residual.index_select(0, rows.long())
+                if pending is not None:
+                    x = x + pending.index_select(0, rows.long())
+            c = x - x.mean(-1, keepdim=True)
+            return (c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight).to(ctx.dtype)
+
+    @register_part("block", "toy_parallel")
+    class ParallelBlock(Block):
+        """x += mixer(n) + feed_forward(n), n = norm(x): one norm, both sub-layers read it, and what
+        they give is handed on as one pending sum for the next norm to add."""
+
+        norm_names = ("input",)
+
+        def __init__(self, mixer, feed_forward, norms, tensors=None):
+            super().__init__(tensors)
+            self.mixer, self.feed_forward, self.norm_in = mixer, feed_forward, norms["input"]
+
+        def children(self):
+            return (self.norm_in, self.mixer, self.feed_forward)
+
+        def forward(self, ctx, residual, delta, cache):
+            n = self.norm_in.forward(ctx, residual, delta)
+            whole = lambda d: d.sum(0) if d.dim() == 3 else d.float()   # planes of a product cut along K
+            return residual, whole(self.mixer.forward(ctx, n, cache)) + whole(self.feed_forward.forward(ctx, n))
+
+    def make_plan(c):
+        h, d = c["hidden_size"], c["head_dim"]
+        centered = lambda name: PartSpec("toy_centered", {"size": h, "eps": c["eps"]}, {"weight": name})
+        rope = PartSpec("rope_neox", {"head_dim": d, "theta": c["theta"]})
+        layers, caches, order = [], [], []
+        for i in range(3):
+            attn = PartSpec("gqa_attention", {"hidden_size": h, "num_heads": c["heads"], "num_kv_heads": c["kv_heads"],
+                                              "head_dim": d, "qk_norm_eps": c["eps"], "position": rope, "window": None},
+                            {k: f"par.{i}.attn.{k}" for k in ("q", "k", "v", "o", "q_norm", "k_norm")})
+            ff = PartSpec("swiglu", {"hidden_size": h, "intermediate_size": c["intermediate_size"]},
+                          {k: f"par.{i}.ff.{k}" for k in ("gate", "up", "down")})
+            layers.append(LayerSpec(PartSpec("toy_parallel"), attn, ff, {"input": centered(f"par.{i}.norm")}))
+            caches.append(CacheSpec("paged_kv", heads=c["kv_heads"], head_dim=d))
+            order.append(RunStep(i, i))
+        sizes = {"vocab_size": c["vocab_size"], "hidden_size": h}
+        return ModelPlan(h, c["vocab_size"], c["max_positions"],
+                         PartSpec("token_embedding", sizes, {"weight": "par.embed"}), layers, caches, order,
+                         centered("par.norm"), PartSpec("linear_head", sizes, {"weight": "par.head"}))
+
+    register_architecture("ToyParallelForCausalLM", dict, make_plan)
+    folder = write_model_folder(tmp_path_factory.mktemp("parallel"), PARALLEL, seed=13, norm_jitter=0.2)
+    yield folder
+    unregister_architecture("ToyParallelForCausalLM")
+    unregister_part("block", "toy_parallel")
+    unregister_part("norm", "toy_centered")
+
+
+def parallel_plain(folder, ids):
+    c, w = P.read_model(folder)
+    t, d, nq, nkv = len(ids), c["head_dim"], c["heads"], c["kv_heads"]
+    pos = torch.arange(t)
+
+    def centered(x, weight):
+        x = x - x.mean(-1, keepdim=True)
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + c["eps"]) * weight
+
+    x = w["par.embed"][torch.as_tensor(ids)]
+    for i in range(3):
+        n, p = centered(x, w[f"par.{i}.norm"]), f"par.{i}.attn"
+        q = P.rope_neox(P.rms_norm((n @ w[f"{p}.q"].T).view(t, nq, d), w[f"{p}.q_norm"], c["eps"]), pos, c["theta"])
+        k = P.rope_neox(P.rms_norm((n @ w[f"{p}.k"].T).view(t, nkv, d), w[f"{p}.k_norm"], c["eps"]), pos, c["theta"])
+        v = (n @ w[f"{p}.v"].T).view(t, nkv, d)
+        ffw = {f"f.{k}_proj.weight": w[f"par.{i}.ff.{k}"] for k in ("gate", "up", "down")}
+        x = x + P.causal_attention(q, k, v) @ w[f"{p}.o"].T + P.feed_forward(n, ffw, "f")
+    return centered(x, w["par.norm"]) @ w["par.head"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail_one_by_one", "portions", "mixed"])
+def test_a_norm_and_a_block_arrangement_of_their_own(parallel_folder, cut, dtype):
+    """A norm that also takes the mean away and a block in which mixer and feed-forward read one
+    normalised input and their outputs are added together, both defined here: registered, built
+    from a plan, loaded, and stepped under every way of cutting (decode steps from HIP graphs:
+    nothing in these parts stands in a capture's way), around the framework's own attention and
+    feed-forward, whose kernels run unchanged."""
+    from qwen3_runtime_amd.config.engine import EngineConfig
+    from qwen3_runtime_amd.engine.factory import load
+
+    reqs = traces.make_requests(PARALLEL["vocab_size"], [70, 9, 41, 33], seed=4)
+    steps = getattr(traces, cut)(reqs)
+    page = 8
+    loaded = load(parallel_folder, EngineConfig(page_size=page, num_pages=-(-traces.peak_tokens(steps, unit=page) // page),
+                                                max_num_seqs=4, dtype=dtype, device=DEV, hip_graph=True))
+    got = traces.replay(loaded, steps)
+    assert loaded.runner.hip_graph and (cut != "tail_one_by_one" or loaded.runner._graphs)
+    want = {(rid, p): row.float() for rid, toks in reqs.items() for p, row in enumerate(parallel_plain(parallel_folder, toks))}
+    if dtype == "float32":
+        traces.compare(got, want, atol=5e-5, rtol=5e-5)
+    else:
+        traces.compare_rounding_noise(got, want)
