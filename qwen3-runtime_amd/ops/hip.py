@@ -631,12 +631,24 @@ class HipOps:
 
     @staticmethod
     def choose_decode_splits(num_tiles: int, nkv: int, max_kv: int) -> int:
-        """Decoding: blocks of four waves; about 256 blocks in all, at least 8 key blocks of 32 each
-        (4 each measured 2 % slower over a batch-1 decode step at 2,048 keys), at most 64 parts
-        (what the merge kernel reads with every load in flight at once)."""
+        """Decoding: blocks of four waves, two to a compute unit. The parts are chosen by a small
+        model of the launch's time that the measurements fit: the busiest compute unit gets
+        ceil(blocks / 256) blocks, each a part of a sequence's keys plus a fixed cost (some 2.5 us:
+        0.06 of a walk over 2,100 keys), so the time goes as ceil(work * parts / 256) *
+        (1 / parts + cost). Counts of blocks that leave some units one block more than others are
+        what it avoids: 12 sequences of 2,100 keys on 8 key heads 32 us in 3 parts (288 blocks), 27
+        in 2; 24 sequences 49 us in 2 parts, 42 in 4; 40 sequences 78 us in 1 part, 65 in 4. At
+        least 8 key blocks of 32 a part (4 each measured 2 % slower over a batch-1 decode step at
+        2,048 keys), at most 64 parts (what the merge kernel reads with every load in flight)."""
         work = num_tiles * nkv
         blocks = (max_kv + 31) // 32
-        return max(1, min((256 + work - 1) // work, blocks // 8, 64))
+        cost = 0.06 * 2100 / max(max_kv, 1)
+        best, best_time = 1, None
+        for parts in range(1, max(1, min(blocks // 8, 64)) + 1):
+            time = -(-work * parts // 256) * (1.0 / parts + cost)
+            if best_time is None or time < best_time * 0.999:
+                best, best_time = parts, time
+        return best
 
     # decoding over unequal lengths: from this ratio of the longest to the mean length on, pieces
     decode_piece_ratio = 1.35
